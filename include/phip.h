@@ -1,0 +1,203 @@
+/*
+ * libphip: C ABI of the MI355X (gfx950) backend for primitiv's matmul path.
+ *
+ * Everything primitiv's `devices::HIP` class needs from the GPU goes through
+ * these entry points: plain pointers and sizes, an int status, no C++ types.
+ * Each declaration names the interface of the reference (primitiv v0.4.0,
+ * paths relative to its root) that it stands behind.
+ *
+ * Conventions
+ *  - Every function returns PHIP_OK (0) or a negative PHIP_ERR_* code and
+ *    never throws.  phip_last_error() returns the calling thread's message
+ *    for the most recent failure.
+ *  - Device pointers are raw HIP device addresses.  Matrices are dense
+ *    column-major (leading dimension = rows); the minibatch is the outermost
+ *    index with stride rows*cols, or stride 0 for an operand whose batch is 1
+ *    (primitiv/devices/eigen/ops/matmul.cc:18-37).
+ *  - All device work of a context is enqueued in order on that context's one
+ *    stream; only the *_d2h copies, phip_sync and phip_event_elapsed_ms block
+ *    the host.  In-order execution is what makes immediate reuse of a pool
+ *    block safe (the reference relies on the same property of the CUDA null
+ *    stream, primitiv/devices/cuda/ops/copy_tensor.cu:20-23).
+ *  - Element types: f32 = float, f16 = IEEE binary16, bf16 = bfloat16.  The
+ *    16-bit variants store 16-bit values and always accumulate in fp32.
+ */
+#ifndef PHIP_H_
+#define PHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PHIP_OK 0
+#define PHIP_ERR_INVALID_ARGUMENT (-1)
+#define PHIP_ERR_RUNTIME (-2)        /* a HIP runtime call failed */
+#define PHIP_ERR_OUT_OF_MEMORY (-3)
+#define PHIP_ERR_UNSUPPORTED (-4)    /* device is not a gfx950 part, etc. */
+
+typedef struct phip_ctx phip_ctx;
+typedef struct phip_event phip_event;
+typedef struct phip_randomizer phip_randomizer;
+
+typedef struct phip_device_info {
+  char name[256];
+  char arch[64];             /* e.g. "gfx950:sramecc+:xnack-" */
+  int32_t device_id;
+  int32_t compute_units;
+  int32_t clock_mhz;         /* peak engine clock */
+  int32_t memory_clock_mhz;
+  int32_t memory_bus_bits;
+  int32_t wavefront_size;
+  int32_t lds_bytes_per_workgroup;
+  int32_t l2_bytes;
+  uint64_t global_memory_bytes;
+} phip_device_info;
+
+/* ---- errors --------------------------------------------------------------
+ * Reference: exceptions `primitiv::Error` raised through PRIMITIV_THROW_ERROR
+ * (primitiv/core/error.h:14-60) and CUDA_CALL (primitiv/internal/cuda/utils.h:
+ * 20-28); the host class turns a non-zero status plus this message into that
+ * exception. */
+const char *phip_last_error(void);
+
+/* ---- devices and contexts -------------------------------------------------
+ * Reference: CUDA::num_devices / assert_support / check_support / ctor / dtor
+ * (primitiv/devices/cuda/device.cu:12-116, primitiv/devices/cuda/device.h:
+ * 27-62) and cuda::InternalState (primitiv/internal/cuda/utils.h:320-350). */
+int phip_device_count(int *count);
+/* PHIP_OK when `device_id` exists, is a gfx950 part and has >= 1 GiB. */
+int phip_check_support(int device_id);
+int phip_ctx_create(int device_id, phip_ctx **out);
+/* Frees every pool block, the stream and the context. */
+int phip_ctx_destroy(phip_ctx *ctx);
+/* Process-unique id of a live context (never reused); 0 is never an id. */
+uint64_t phip_ctx_id(const phip_ctx *ctx);
+int phip_device_info_get(phip_ctx *ctx, phip_device_info *out);
+/* Writes the human-readable description used by Device::dump_description
+ * (primitiv/devices/cuda/ops/dump_description.cu:12-40) into buf. */
+int phip_describe(phip_ctx *ctx, char *buf, size_t buf_size);
+int phip_sync(phip_ctx *ctx);
+
+/* ---- raw memory -----------------------------------------------------------
+ * Reference: the allocator / deleter lambdas handed to MemoryPool
+ * (primitiv/internal/cuda/utils.h:330-340).  phip_malloc fails with
+ * PHIP_ERR_OUT_OF_MEMORY so the caller's pool can release blocks and retry
+ * (primitiv/core/memory_pool.cc:53-63). */
+int phip_malloc(phip_ctx *ctx, size_t bytes, void **out);
+int phip_free(phip_ctx *ctx, void *ptr);
+
+/* ---- pooled memory --------------------------------------------------------
+ * Reference: MemoryPool::allocate / free / release_reserved_blocks
+ * (primitiv/core/memory_pool.cc:35-95): request rounded up to a power of two
+ * (at least `2*sizeof(float)`, primitiv/internal/cuda/utils.h:337-342),
+ * per-size free lists, one retry after releasing the reserved blocks.
+ * bytes == 0 yields *out = NULL, *allocated = 0. */
+int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated);
+int phip_pool_free(phip_ctx *ctx, void *ptr);
+/* Same as phip_pool_free but addressed by context id; succeeds silently when
+ * that context is already destroyed (its memory went with it).  This is the
+ * deleter of a tensor handle that may outlive its device
+ * (primitiv/core/memory_pool.h:22-35, test/cuda_device_test.cc:66-78). */
+int phip_pool_free_by_id(uint64_t ctx_id, void *ptr);
+int phip_pool_release_reserved(phip_ctx *ctx);
+/* Bytes currently handed out / held in free lists. */
+int phip_pool_stats(phip_ctx *ctx, uint64_t *supplied_bytes, uint64_t *reserved_bytes);
+
+/* ---- copies ---------------------------------------------------------------
+ * Reference: reset_tensor_by_array_impl (primitiv/devices/cuda/ops/
+ * reset_tensor_by_array.cu:10-15), tensor_to_vector_impl (.../tensor_to_vector.cu:
+ * 10-17), copy_tensor_impl (.../copy_tensor.cu:10-30).  h2d returns when the
+ * host buffer may be reused; d2h returns when the data has arrived. */
+int phip_memcpy_h2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes);
+int phip_memcpy_d2h(phip_ctx *ctx, void *dst, const void *src, size_t bytes);
+int phip_memcpy_d2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes);
+
+/* ---- fill and storage conversion -----------------------------------------
+ * Reference: reset_tensor_impl (primitiv/devices/cuda/ops/reset_tensor.cu:9-24,
+ * primitiv/devices/cuda16/ops/reset_tensor.cu:9-24) and the fp32<->fp16 staging
+ * kernels of the half-storage device (primitiv/devices/cuda16/ops/
+ * reset_tensor_by_array.cu:9-30, .../tensor_to_vector.cu:9-32).
+ * Conversions round to nearest even. */
+int phip_fill_f32(phip_ctx *ctx, float *p, float value, size_t n);
+int phip_fill_f16(phip_ctx *ctx, void *p, float value, size_t n);
+int phip_fill_bf16(phip_ctx *ctx, void *p, float value, size_t n);
+int phip_cvt_f32_to_f16(phip_ctx *ctx, const float *src, void *dst, size_t n);
+int phip_cvt_f16_to_f32(phip_ctx *ctx, const void *src, float *dst, size_t n);
+int phip_cvt_f32_to_bf16(phip_ctx *ctx, const float *src, void *dst, size_t n);
+int phip_cvt_bf16_to_f32(phip_ctx *ctx, const void *src, float *dst, size_t n);
+
+/* ---- y += x with minibatch broadcasting ------------------------------------
+ * Reference: inplace_add_impl (primitiv/devices/eigen/ops/inplace_add.cc:9-23,
+ * primitiv/devices/cuda/ops/inplace_add.cu:9-30, .../cuda16/ops/inplace_add.cu:
+ * 9-40).  x holds `volume*bx` elements, y `volume*by`; bx == by, or one of
+ * them is 1.  by == 1 < bx adds the sum of x over the minibatch. */
+int phip_inplace_add_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bx, uint32_t by);
+int phip_inplace_add_f16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by);
+int phip_inplace_add_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by);
+
+/* ---- y[i] = sum over the minibatch of x[n][i] ------------------------------
+ * Reference: batch_sum_fw_impl (primitiv/devices/eigen/ops/batch_sum.cc:9-22,
+ * primitiv/devices/cuda/ops/batch_sum.cu:9-33, .../cuda16/ops/batch_sum.cu:9-33). */
+int phip_batch_sum_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bs);
+int phip_batch_sum_f16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bs);
+int phip_batch_sum_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bs);
+
+/* ---- matmul forward:  y = a . b  per sample --------------------------------
+ * Reference: Device::matmul_fw_impl (primitiv/core/device.h:464;
+ * primitiv/devices/eigen/ops/matmul.cc:9-38; primitiv/devices/cuda/ops/matmul.cu:
+ * 21-66; primitiv/devices/cuda16/ops/matmul.cu:46-126).
+ * a: [di x dj] x ba, b: [dj x dk] x bb, y: [di x dk] x max(ba, bb); ba == bb
+ * or one of them is 1.  y is overwritten and may be uninitialised on entry. */
+int phip_matmul_fw_f32(phip_ctx *ctx, const float *a, const float *b, float *y,
+                       uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+int phip_matmul_fw_f16(phip_ctx *ctx, const void *a, const void *b, void *y,
+                       uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+int phip_matmul_fw_bf16(phip_ctx *ctx, const void *a, const void *b, void *y,
+                        uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+
+/* ---- matmul backward:  ga += gy . b^T ,  gb += a^T . gy --------------------
+ * Reference: Device::matmul_bw_impl (primitiv/core/device.h:481-483;
+ * primitiv/devices/eigen/ops/matmul.cc:40-79; primitiv/devices/cuda/ops/matmul.cu:
+ * 68-139; primitiv/devices/cuda16/ops/matmul.cu:128-266).
+ * Both gradients are accumulated into.  The gradient of an operand whose
+ * batch is 1 is reduced over the minibatch inside the kernel (the reference's
+ * CUDA device issues one GEMM per sample for that case, matmul.cu:113-123). */
+int phip_matmul_bw_f32(phip_ctx *ctx, const float *a, const float *b, const float *gy,
+                       float *ga, float *gb,
+                       uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+int phip_matmul_bw_f16(phip_ctx *ctx, const void *a, const void *b, const void *gy,
+                       void *ga, void *gb,
+                       uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+int phip_matmul_bw_bf16(phip_ctx *ctx, const void *a, const void *b, const void *gy,
+                        void *ga, void *gb,
+                        uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+
+/* ---- timing ---------------------------------------------------------------
+ * No counterpart in the reference (it has no profiling facility); events are
+ * recorded on the context's stream so they bracket exactly the kernels the
+ * library launched. */
+int phip_event_create(phip_ctx *ctx, phip_event **out);
+int phip_event_destroy(phip_event *ev);
+int phip_event_record(phip_ctx *ctx, phip_event *ev);
+/* Waits for `stop`, then returns the milliseconds between the two events. */
+int phip_event_elapsed_ms(phip_event *start, phip_event *stop, float *ms);
+
+/* ---- host-side seeded inputs ----------------------------------------------
+ * Reference: DefaultRandomizer (primitiv/core/random.h:15-87), the generator
+ * behind the CPU devices' random_* ops: std::mt19937 with one freshly built
+ * standard-library distribution per fill.  uniform yields (lower, upper].
+ * These run on the host and write host memory; they exist so that every
+ * device is handed bit-identical seeded inputs. */
+int phip_randomizer_create(uint32_t seed, phip_randomizer **out);
+int phip_randomizer_destroy(phip_randomizer *r);
+int phip_randomizer_fill_uniform(phip_randomizer *r, float lower, float upper, size_t n, float *host_out);
+int phip_randomizer_fill_normal(phip_randomizer *r, float mean, float sd, size_t n, float *host_out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PHIP_H_ */

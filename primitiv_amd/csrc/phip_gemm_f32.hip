@@ -1,0 +1,390 @@
+// fp32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// One workgroup of 256 threads (4 wavefronts) owns a BM x BN tile of C and
+// walks K in steps of BK.  Operand tiles are staged through LDS in a common
+// [k][m] / [k][n] layout whatever their layout in memory: an operand that is
+// contiguous along m (or n) is copied row by row with 16-byte accesses, one
+// that is contiguous along k is transposed while it is written to LDS.  The
+// three products of primitiv's matmul (a.b, gy.b^T, a^T.gy) are therefore the
+// same inner loop behind different loaders, and no transposed copy of any
+// operand is ever materialised.
+//
+// Two LDS stages: the loads of tile t+1 are issued before the matrix
+// instructions of tile t and written to the other stage afterwards, with one
+// barrier per tile.
+#include "phip_internal.h"
+
+namespace phip {
+namespace {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kPad = 4;  // floats appended to every LDS row
+
+struct GemmArgs {
+  const float *A;
+  const float *B;
+  float *C;
+  int M, N, K;
+  long lda, ldb, ldc;
+  long sA, sB, sC;
+  long rA, rB;
+  int tiles_m, tiles_n;
+  int splits;        // workgroups that share one C tile, each taking a K range
+  int ktiles_per_r;  // ceil(K / BK)
+  int total_ktiles;  // rbatch * ktiles_per_r
+  int atomic;        // 1: add the tile into C with atomics (split K)
+  int accumulate;    // 1: C += tile, 0: C = tile (ignored when atomic)
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
+// Renumber them so that one XCD receives a contiguous run of tiles.
+__device__ inline int xcd_remap(int bid, int total) {
+  constexpr int kXcds = 8;
+  const int xcd = bid % kXcds;
+  const int idx = bid / kXcds;
+  const int q = total / kXcds, rem = total % kXcds;
+  return xcd * q + (xcd < rem ? xcd : rem) + idx;
+}
+
+// Tile of an operand that is contiguous along x (m or n): element (x, k) at
+// base[x + k*ld].  Rows of the LDS tile are k.
+template <int BX, int BK, int V>
+struct LoaderXContig {
+  static constexpr int kVecPerRow = BX / V;
+  static constexpr int kTotal = BX * BK / V;
+  static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
+  float regs[kIters][V];
+
+  __device__ inline void load(const float *base, long ld, int x0, int X, int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      const int k = k0 + v / kVecPerRow;
+      const int x = x0 + (v % kVecPerRow) * V;
+      const bool live = (kTotal % kThreads == 0 || v < kTotal) && k < K;
+      if (V == 4 && live && x + 4 <= X) {
+        const float4v t = *reinterpret_cast<const float4v *>(base + x + (long)k * ld);
+        regs[i][0] = t.x; regs[i][1 % V] = t.y; regs[i][2 % V] = t.z; regs[i][3 % V] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          regs[i][e] = (live && x + e < X) ? base[x + e + (long)k * ld] : 0.0f;
+        }
+      }
+    }
+  }
+
+  __device__ inline void store(float *lds, int tid) const {
+    constexpr int S = BX + kPad;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      float *p = lds + (v / kVecPerRow) * S + (v % kVecPerRow) * V;
+      if (V == 4) {
+        float4v t = {regs[i][0], regs[i][1 % V], regs[i][2 % V], regs[i][3 % V]};
+        *reinterpret_cast<float4v *>(p) = t;
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) p[e] = regs[i][e];
+      }
+    }
+  }
+};
+
+// Tile of an operand that is contiguous along k: element (x, k) at
+// base[k + x*ld].  Transposed on its way into LDS.
+template <int BX, int BK, int V>
+struct LoaderKContig {
+  static constexpr int kVecPerX = BK / V;
+  static constexpr int kTotal = BX * BK / V;
+  static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
+  float regs[kIters][V];
+
+  __device__ inline void load(const float *base, long ld, int x0, int X, int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      const int x = x0 + v / kVecPerX;
+      const int k = k0 + (v % kVecPerX) * V;
+      const bool live = (kTotal % kThreads == 0 || v < kTotal) && x < X;
+      if (V == 4 && live && k + 4 <= K) {
+        const float4v t = *reinterpret_cast<const float4v *>(base + k + (long)x * ld);
+        regs[i][0] = t.x; regs[i][1 % V] = t.y; regs[i][2 % V] = t.z; regs[i][3 % V] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          regs[i][e] = (live && k + e < K) ? base[k + e + (long)x * ld] : 0.0f;
+        }
+      }
+    }
+  }
+
+  __device__ inline void store(float *lds, int tid) const {
+    constexpr int S = BX + kPad;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      float *p = lds + ((v % kVecPerX) * V) * S + v / kVecPerX;
+#pragma unroll
+      for (int e = 0; e < V; ++e) p[e * S] = regs[i][e];
+    }
+  }
+};
+
+template <bool KMAJOR, int BX, int BK, int V>
+struct LoaderSelect {
+  typedef LoaderXContig<BX, BK, V> type;
+};
+template <int BX, int BK, int V>
+struct LoaderSelect<true, BX, BK, V> {
+  typedef LoaderKContig<BX, BK, V> type;
+};
+
+// WGM x WGN x WGK wavefronts: WGM*WGN of them tile the BM x BN block, WGK of
+// them share each wave tile and split the k steps of every K tile between
+// themselves (their partial tiles are summed through LDS at the end).
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool A_KMAJOR, bool B_KMAJOR, int V>
+__global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const GemmArgs g) {
+  static_assert(WGM * WGN * WGK == 4, "four wavefronts per workgroup");
+  constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 blocks");
+  static_assert((BK / 2) % WGK == 0, "k steps must divide among the k-split waves");
+  constexpr int SA = BM + kPad, SB = BN + kPad;
+  constexpr int kStageA = BK * SA, kStageB = BK * SB;
+  constexpr int kTileFloats = 2 * (kStageA + kStageB);
+  constexpr int kReduceFloats = WGK > 1 ? 4 * TM * TN * 16 * 64 : 0;
+  constexpr int kLdsFloats = kTileFloats > kReduceFloats ? kTileFloats : kReduceFloats;
+  __shared__ __attribute__((aligned(16))) float lds[kLdsFloats];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wk = wave % WGK;
+  const int wm = (wave / WGK) % WGM;
+  const int wn = (wave / WGK) / WGM;
+
+  int t = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
+  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
+  const int split = t % g.splits;
+  const int z = t / g.splits;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int kt_begin = (int)((long)split * g.total_ktiles / g.splits);
+  const int kt_end = (int)((long)(split + 1) * g.total_ktiles / g.splits);
+
+  const float *Az = g.A + (long)z * g.sA;
+  const float *Bz = g.B + (long)z * g.sB;
+
+  typename LoaderSelect<A_KMAJOR, BM, BK, V>::type la;
+  typename LoaderSelect<B_KMAJOR, BN, BK, V>::type lb;
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  auto fetch = [&](int kt) {
+    const int r = kt / g.ktiles_per_r;
+    const int k0 = (kt - r * g.ktiles_per_r) * BK;
+    la.load(Az + (long)r * g.rA, g.lda, m0, g.M, k0, g.K, tid);
+    lb.load(Bz + (long)r * g.rB, g.ldb, n0, g.N, k0, g.K, tid);
+  };
+
+  if (kt_begin < kt_end) {
+    fetch(kt_begin);
+    la.store(lds, tid);
+    lb.store(lds + 2 * kStageA, tid);
+  }
+  __syncthreads();
+
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int stage = (kt - kt_begin) & 1;
+    const bool more = kt + 1 < kt_end;
+    if (more) fetch(kt + 1);
+
+    const float *as = lds + stage * kStageA + wm * WTM + (lane & 31);
+    const float *bs = lds + 2 * kStageA + stage * kStageB + wn * WTN + (lane & 31);
+    const int khalf = lane >> 5;
+#pragma unroll
+    for (int s = 0; s < BK / 2 / WGK; ++s) {
+      const int kk = (s * WGK + wk) * 2 + khalf;
+      float af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = as[kk * SA + i * 32];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = bs[kk * SB + j * 32];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          // rows of the instruction's result follow n, its columns follow m
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+
+    if (more) {
+      la.store(lds + (stage ^ 1) * kStageA, tid);
+      lb.store(lds + 2 * kStageA + (stage ^ 1) * kStageB, tid);
+    }
+    __syncthreads();
+  }
+
+  // Lane l of result register v holds C(m, n) with m = l % 32 and
+  // n = 8*(v/4) + 4*(l/32) + v%4 inside its 32x32 block.
+  float *Cz = g.C + (long)z * g.sC;
+  const int cm = m0 + wm * WTM + (lane & 31);
+  const int cn = n0 + wn * WTN + 4 * (lane >> 5);
+
+  if (WGK > 1) {
+    // Sum the k-split waves' tiles: every wave parks its registers in LDS,
+    // then wave w reduces and writes registers [4w, 4w+4) of each block.
+    float *red = lds;  // the tile stages are no longer read (barrier above)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          red[(((wave * TM + i) * TN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+    __syncthreads();
+    const int group = wave / WGK;  // waves of one group share a wave tile
+    constexpr int kPer = 16 / WGK;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+          const int v = wk * kPer + q;
+          float s = 0.0f;
+#pragma unroll
+          for (int w = 0; w < WGK; ++w)
+            s += red[((((group * WGK + w) * TM + i) * TN + j) * 16 + v) * 64 + lane];
+          const int m = cm + i * 32;
+          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
+          if (m < g.M && n < g.N) {
+            float *p = Cz + m + (long)n * g.ldc;
+            if (g.atomic) unsafeAtomicAdd(p, s);
+            else *p = g.accumulate ? *p + s : s;
+          }
+        }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = cm + i * 32;
+          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
+          if (m < g.M && n < g.N) {
+            float *p = Cz + m + (long)n * g.ldc;
+            const float s = acc[i][j][v];
+            if (g.atomic) unsafeAtomicAdd(p, s);
+            else *p = g.accumulate ? *p + s : s;
+          }
+        }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void zero_c_kernel(float *C, int M, int N, long ldc, long sC, int batch) {
+  const long per = (long)M * N;
+  const long total = per * batch;
+  for (long i = (long)blockIdx.x * kThreads + threadIdx.x; i < total; i += (long)gridDim.x * kThreads) {
+    const long z = i / per, e = i - z * per;
+    C[z * sC + (e % M) + (e / M) * ldc] = 0.0f;
+  }
+}
+
+struct TileChoice {
+  int bm, bn, bk;
+};
+
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK>
+int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec4) {
+  a.tiles_m = (p.M + BM - 1) / BM;
+  a.tiles_n = (p.N + BN - 1) / BN;
+  a.ktiles_per_r = (p.K + BK - 1) / BK;
+  a.total_ktiles = a.ktiles_per_r * p.rbatch;
+  const long tiles = (long)a.tiles_m * a.tiles_n * p.batch;
+
+  // Split K between workgroups when the C tiles alone cannot fill the chip.
+  const int cus = ctx->prop.multiProcessorCount;
+  int splits = 1;
+  if (tiles < 2 * cus) {
+    const long want = (4L * cus + tiles - 1) / tiles;
+    const int min_ktiles = BK >= 64 ? 2 : 4;  // K tiles per workgroup worth a launch
+    long cap = a.total_ktiles / min_ktiles;
+    if (cap < 1) cap = 1;
+    splits = (int)(want < cap ? want : cap);
+  }
+  a.splits = splits;
+  a.atomic = splits > 1;
+  const long grid = tiles * splits;
+  if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
+
+  if (a.atomic && !p.accumulate) {
+    const long total = (long)p.M * p.N * p.batch;
+    long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+    if (blocks > cus * 8L) blocks = cus * 8L;
+    hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream,
+                       a.C, p.M, p.N, p.ldc, p.sC, p.batch);
+    PHIP_LAUNCH_CHECK();
+  }
+
+#define PHIP_LAUNCH(AK, BKM, VV)                                                                   \
+  hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VV>), dim3((unsigned)grid), \
+                     dim3(kThreads), 0, ctx->stream, a)
+  if (!p.a_kmajor && p.b_kmajor) {
+    if (vec4) PHIP_LAUNCH(false, true, 4); else PHIP_LAUNCH(false, true, 1);
+  } else if (!p.a_kmajor && !p.b_kmajor) {
+    if (vec4) PHIP_LAUNCH(false, false, 4); else PHIP_LAUNCH(false, false, 1);
+  } else if (p.a_kmajor && p.b_kmajor) {
+    if (vec4) PHIP_LAUNCH(true, true, 4); else PHIP_LAUNCH(true, true, 1);
+  } else {
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
+  }
+#undef PHIP_LAUNCH
+  PHIP_LAUNCH_CHECK();
+  return PHIP_OK;
+}
+
+}  // namespace
+
+int gemm_f32(phip_ctx *ctx, const Gemm &p) {
+  if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return PHIP_OK;
+  GemmArgs a;
+  a.A = static_cast<const float *>(p.A);
+  a.B = static_cast<const float *>(p.B);
+  a.C = static_cast<float *>(p.C);
+  a.M = p.M; a.N = p.N; a.K = p.K;
+  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
+  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
+  a.rA = p.rA; a.rB = p.rB;
+  a.accumulate = p.accumulate ? 1 : 0;
+  a.atomic = 0;
+
+  auto aligned = [](const void *ptr, long ld, long s, long r) {
+    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
+  };
+  const bool vec4 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB);
+
+  const int cus = ctx->prop.multiProcessorCount;
+  auto tiles = [&](int bm, int bn) {
+    return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch;
+  };
+  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1>(ctx, p, a, vec4);
+  if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1>(ctx, p, a, vec4);
+  return launch_tile<32, 32, 64, 1, 1, 4>(ctx, p, a, vec4);
+}
+
+}  // namespace phip

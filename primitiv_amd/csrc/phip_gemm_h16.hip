@@ -1,0 +1,364 @@
+// GEMM for 16-bit storage (fp16 or bf16) with fp32 accumulation on the gfx950
+// matrix cores (v_mfma_f32_32x32x16_f16 / _bf16).
+//
+// Same workgroup structure as the fp32 kernel, but the matrix instruction
+// wants 8 consecutive k values per lane, so the common LDS layout is [m][k] /
+// [n][k]: an operand that is contiguous along k in memory is copied with
+// 16-byte accesses, one that is contiguous along m or n is transposed while it
+// is written to LDS.  Results are rounded to the storage type once, after the
+// whole K range has been accumulated in fp32; `C += ...` reads C, adds in fp32
+// and rounds once.
+#include "phip_internal.h"
+#include "phip_types.h"
+
+namespace phip {
+namespace {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kPadH = 8;  // 16-bit elements appended to every LDS row
+
+struct GemmArgsH {
+  const uint16_t *A;
+  const uint16_t *B;
+  uint16_t *C;
+  int M, N, K;
+  long lda, ldb, ldc;
+  long sA, sB, sC;
+  long rA, rB;
+  int tiles_m, tiles_n;
+  int ktiles_per_r;
+  int total_ktiles;
+  int accumulate;
+};
+
+__device__ inline int xcd_remap(int bid, int total) {
+  constexpr int kXcds = 8;
+  const int xcd = bid % kXcds;
+  const int idx = bid / kXcds;
+  const int q = total / kXcds, rem = total % kXcds;
+  return xcd * q + (xcd < rem ? xcd : rem) + idx;
+}
+
+union Pack8 {
+  uint4v v;
+  uint16_t h[8];
+};
+
+// Operand contiguous along k: element (x, k) at base[k + x*ld]; LDS rows are x.
+template <int BX, int BK, int V>
+struct LoaderKContigH {
+  static constexpr int kVecPerX = BK / V;
+  static constexpr int kTotal = BX * BK / V;
+  static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
+  Pack8 regs[kIters];
+
+  __device__ inline void load(const uint16_t *base, long ld, int x0, int X, int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      const int x = x0 + v / kVecPerX;
+      const int k = k0 + (v % kVecPerX) * V;
+      const bool live = (kTotal % kThreads == 0 || v < kTotal) && x < X;
+      if (V == 8 && live && k + 8 <= K) {
+        regs[i].v = *reinterpret_cast<const uint4v *>(base + k + (long)x * ld);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) regs[i].h[e] = (live && k + e < K) ? base[k + e + (long)x * ld] : (uint16_t)0;
+      }
+    }
+  }
+
+  __device__ inline void store(uint16_t *lds, int tid) const {
+    constexpr int S = BK + kPadH;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      uint16_t *p = lds + (v / kVecPerX) * S + (v % kVecPerX) * V;
+      if (V == 8) {
+        *reinterpret_cast<uint4v *>(p) = regs[i].v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) p[e] = regs[i].h[e];
+      }
+    }
+  }
+};
+
+// Operand contiguous along x: element (x, k) at base[x + k*ld]; transposed on
+// its way into LDS.
+template <int BX, int BK, int V>
+struct LoaderXContigH {
+  static constexpr int kVecPerRow = BX / V;
+  static constexpr int kTotal = BX * BK / V;
+  static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
+  Pack8 regs[kIters];
+
+  __device__ inline void load(const uint16_t *base, long ld, int x0, int X, int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      const int k = k0 + v / kVecPerRow;
+      const int x = x0 + (v % kVecPerRow) * V;
+      const bool live = (kTotal % kThreads == 0 || v < kTotal) && k < K;
+      if (V == 8 && live && x + 8 <= X) {
+        regs[i].v = *reinterpret_cast<const uint4v *>(base + x + (long)k * ld);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) regs[i].h[e] = (live && x + e < X) ? base[x + e + (long)k * ld] : (uint16_t)0;
+      }
+    }
+  }
+
+  __device__ inline void store(uint16_t *lds, int tid) const {
+    constexpr int S = BK + kPadH;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int v = tid + i * kThreads;
+      if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      uint16_t *p = lds + ((v % kVecPerRow) * V) * S + v / kVecPerRow;
+#pragma unroll
+      for (int e = 0; e < V; ++e) p[e * S] = regs[i].h[e];
+    }
+  }
+};
+
+template <bool KMAJOR, int BX, int BK, int V>
+struct LoaderSelectH {
+  typedef LoaderXContigH<BX, BK, V> type;
+};
+template <int BX, int BK, int V>
+struct LoaderSelectH<true, BX, BK, V> {
+  typedef LoaderKContigH<BX, BK, V> type;
+};
+
+template <bool BF16>
+__device__ inline float16v mfma_32x32x16(uint4v a, uint4v b, float16v c) {
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, a), __builtin_bit_cast(half8v, b), c, 0, 0, 0);
+  }
+}
+
+template <bool BF16>
+__device__ inline float load_c(const uint16_t *p) {
+  if constexpr (BF16) {
+    bf16_t t; t.bits = *p; return to_f32(t);
+  } else {
+    return to_f32(__builtin_bit_cast(f16_t, *p));
+  }
+}
+
+template <bool BF16>
+__device__ inline uint16_t round_c(float x) {
+  if constexpr (BF16) {
+    return from_f32<bf16_t>(x).bits;
+  } else {
+    return __builtin_bit_cast(uint16_t, from_f32<f16_t>(x));
+  }
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool A_KMAJOR, bool B_KMAJOR, int V, bool BF16>
+__global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
+  static_assert(WGM * WGN * WGK == 4, "four wavefronts per workgroup");
+  constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 blocks");
+  static_assert((BK / 16) % WGK == 0, "k steps must divide among the k-split waves");
+  constexpr int S = BK + kPadH;  // LDS row stride in 16-bit elements
+  constexpr int kStageA = BM * S, kStageB = BN * S;
+  constexpr int kTileBytes = 2 * (kStageA + kStageB) * 2;
+  constexpr int kReduceBytes = WGK > 1 ? 4 * TM * TN * 16 * 64 * 4 : 0;
+  constexpr int kLdsBytes = kTileBytes > kReduceBytes ? kTileBytes : kReduceBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
+  uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wk = wave % WGK;
+  const int wm = (wave / WGK) % WGM;
+  const int wn = (wave / WGK) / WGM;
+
+  int t = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
+  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
+  const int z = t;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const uint16_t *Az = g.A + (long)z * g.sA;
+  const uint16_t *Bz = g.B + (long)z * g.sB;
+
+  typename LoaderSelectH<A_KMAJOR, BM, BK, V>::type la;
+  typename LoaderSelectH<B_KMAJOR, BN, BK, V>::type lb;
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  auto fetch = [&](int kt) {
+    const int r = kt / g.ktiles_per_r;
+    const int k0 = (kt - r * g.ktiles_per_r) * BK;
+    la.load(Az + (long)r * g.rA, g.lda, m0, g.M, k0, g.K, tid);
+    lb.load(Bz + (long)r * g.rB, g.ldb, n0, g.N, k0, g.K, tid);
+  };
+
+  const int kt_end = g.total_ktiles;
+  if (kt_end > 0) {
+    fetch(0);
+    la.store(lds, tid);
+    lb.store(lds + 2 * kStageA, tid);
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < kt_end; ++kt) {
+    const int stage = kt & 1;
+    const bool more = kt + 1 < kt_end;
+    if (more) fetch(kt + 1);
+
+    // lane l supplies row l%32 and the 8 k values starting at 8*(l/32)
+    const uint16_t *as = lds + stage * kStageA + (wm * WTM + (lane & 31)) * S + 8 * (lane >> 5);
+    const uint16_t *bs = lds + 2 * kStageA + stage * kStageB + (wn * WTN + (lane & 31)) * S + 8 * (lane >> 5);
+#pragma unroll
+    for (int s = 0; s < BK / 16 / WGK; ++s) {
+      const int kk = (s * WGK + wk) * 16;
+      uint4v af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4v *>(as + i * 32 * S + kk);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const uint4v *>(bs + j * 32 * S + kk);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16<BF16>(bf[j], af[i], acc[i][j]);
+    }
+
+    if (more) {
+      la.store(lds + (stage ^ 1) * kStageA, tid);
+      lb.store(lds + 2 * kStageA + (stage ^ 1) * kStageB, tid);
+    }
+    __syncthreads();
+  }
+
+  uint16_t *Cz = g.C + (long)z * g.sC;
+  const int cm = m0 + wm * WTM + (lane & 31);
+  const int cn = n0 + wn * WTN + 4 * (lane >> 5);
+
+  if (WGK > 1) {
+    float *red = reinterpret_cast<float *>(lds_raw);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          red[(((wave * TM + i) * TN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+    __syncthreads();
+    const int group = wave / WGK;
+    constexpr int kPer = 16 / WGK;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+          const int v = wk * kPer + q;
+          float s = 0.0f;
+#pragma unroll
+          for (int w = 0; w < WGK; ++w)
+            s += red[((((group * WGK + w) * TM + i) * TN + j) * 16 + v) * 64 + lane];
+          const int m = cm + i * 32;
+          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
+          if (m < g.M && n < g.N) {
+            uint16_t *p = Cz + m + (long)n * g.ldc;
+            *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+          }
+        }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = cm + i * 32;
+          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
+          if (m < g.M && n < g.N) {
+            uint16_t *p = Cz + m + (long)n * g.ldc;
+            const float s = acc[i][j][v];
+            *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+          }
+        }
+  }
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool BF16>
+int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8) {
+  a.tiles_m = (p.M + BM - 1) / BM;
+  a.tiles_n = (p.N + BN - 1) / BN;
+  a.ktiles_per_r = (p.K + BK - 1) / BK;
+  a.total_ktiles = a.ktiles_per_r * p.rbatch;
+  const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
+  if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
+
+#define PHIP_LAUNCH(AK, BKM, VV)                                                                          \
+  hipLaunchKernelGGL((gemm_h16_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VV, BF16>), dim3((unsigned)grid), \
+                     dim3(kThreads), 0, ctx->stream, a)
+  if (!p.a_kmajor && p.b_kmajor) {
+    if (vec8) PHIP_LAUNCH(false, true, 8); else PHIP_LAUNCH(false, true, 1);
+  } else if (!p.a_kmajor && !p.b_kmajor) {
+    if (vec8) PHIP_LAUNCH(false, false, 8); else PHIP_LAUNCH(false, false, 1);
+  } else if (p.a_kmajor && p.b_kmajor) {
+    if (vec8) PHIP_LAUNCH(true, true, 8); else PHIP_LAUNCH(true, true, 1);
+  } else {
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
+  }
+#undef PHIP_LAUNCH
+  PHIP_LAUNCH_CHECK();
+  return PHIP_OK;
+}
+
+template <bool BF16>
+int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
+  GemmArgsH a;
+  a.A = static_cast<const uint16_t *>(p.A);
+  a.B = static_cast<const uint16_t *>(p.B);
+  a.C = static_cast<uint16_t *>(p.C);
+  a.M = p.M; a.N = p.N; a.K = p.K;
+  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
+  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
+  a.rA = p.rA; a.rB = p.rB;
+  a.accumulate = p.accumulate ? 1 : 0;
+
+  auto aligned = [](const void *ptr, long ld, long s, long r) {
+    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 8 == 0 && s % 8 == 0 && r % 8 == 0;
+  };
+  const bool vec8 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB);
+
+  const int cus = ctx->prop.multiProcessorCount;
+  auto tiles = [&](int bm, int bn) {
+    return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch;
+  };
+  if (tiles(128, 128) >= cus) return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
+  if (tiles(64, 64) >= cus) return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
+  return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec8);
+}
+
+}  // namespace
+
+int gemm_h16(phip_ctx *ctx, const Gemm &p, Elem elem) {
+  if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return PHIP_OK;
+  return elem == Elem::BF16 ? gemm_h16_typed<true>(ctx, p) : gemm_h16_typed<false>(ctx, p);
+}
+
+}  // namespace phip

@@ -1,0 +1,102 @@
+// Internal declarations shared by the translation units of libphip.
+#ifndef PHIP_INTERNAL_H_
+#define PHIP_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/phip.h"
+
+namespace phip {
+
+// Records the calling thread's error message and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Power-of-two bucketed device memory pool (one per context).
+struct Pool {
+  std::vector<std::vector<void *>> reserved{64};
+  std::unordered_map<void *, unsigned> supplied;
+  static constexpr size_t kMinimumSize = 2 * sizeof(float);
+};
+
+}  // namespace phip
+
+struct phip_ctx {
+  int device = -1;
+  uint64_t id = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t prop;
+  phip::Pool pool;
+  std::mutex mutex;  // guards `pool`
+};
+
+struct phip_event {
+  hipEvent_t ev = nullptr;
+  int device = -1;
+};
+
+#define PHIP_HIP(expr)                                                        \
+  do {                                                                        \
+    hipError_t phip_err__ = (expr);                                           \
+    if (phip_err__ != hipSuccess) {                                           \
+      return phip::fail(phip_err__ == hipErrorOutOfMemory                     \
+                            ? PHIP_ERR_OUT_OF_MEMORY                          \
+                            : PHIP_ERR_RUNTIME,                               \
+                        "%s failed: %s (%s:%d)", #expr,                       \
+                        hipGetErrorString(phip_err__), __FILE__, __LINE__);   \
+    }                                                                         \
+  } while (0)
+
+#define PHIP_REQUIRE(cond, ...)                                               \
+  do {                                                                        \
+    if (!(cond)) return phip::fail(PHIP_ERR_INVALID_ARGUMENT, __VA_ARGS__);   \
+  } while (0)
+
+// Makes the context's device current and checks the context pointer.
+#define PHIP_ENTER(ctx)                                                       \
+  PHIP_REQUIRE((ctx) != nullptr, "null context");                             \
+  PHIP_HIP(hipSetDevice((ctx)->device))
+
+// Checks the status of the launch that was just enqueued.
+#define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
+
+namespace phip {
+
+// ---- GEMM layer (phip_gemm_*.hip) ------------------------------------------
+//
+// One problem:  C[z] (M x N, column-major, ldc)  (=|+=)
+//                 sum_{r < rbatch} opA[z][r] (M x K) . opB[z][r] (K x N)
+// for z < batch.  Operand element (m, k) of opA lives at
+//   A + z*sA + r*rA + (a_kmajor ? k + m*lda : m + k*lda)
+// and element (k, n) of opB at
+//   B + z*sB + r*rB + (b_kmajor ? k + n*ldb : n + k*ldb).
+// Strides are in elements and may be 0.
+struct Gemm {
+  int M = 0, N = 0, K = 0;
+  const void *A = nullptr;
+  const void *B = nullptr;
+  void *C = nullptr;
+  long lda = 0, ldb = 0, ldc = 0;
+  long sA = 0, sB = 0, sC = 0;  // per-z strides
+  long rA = 0, rB = 0;          // per-r strides (reduction over samples)
+  int batch = 1;
+  int rbatch = 1;
+  bool a_kmajor = false;  // false: M-contiguous, true: K-contiguous
+  bool b_kmajor = true;   // true: K-contiguous, false: N-contiguous
+  bool accumulate = false;
+};
+
+enum class Elem { F32, F16, BF16 };
+
+int gemm_f32(phip_ctx *ctx, const Gemm &g);
+int gemm_h16(phip_ctx *ctx, const Gemm &g, Elem elem);
+
+}  // namespace phip
+
+#endif  // PHIP_INTERNAL_H_

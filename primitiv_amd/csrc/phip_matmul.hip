@@ -1,0 +1,152 @@
+// primitiv's matmul forward / backward expressed as GEMM problems.
+//
+// a: [di x dj] x ba, b: [dj x dk] x bb, y: [di x dk] x max(ba, bb), all dense
+// column-major with the minibatch outermost.  Four batch cases:
+//
+//   ba == 1 (b shared or not): the minibatch of b is folded into its columns,
+//       so forward, gA and gB are ONE product each with n or k = dk*bb.  For
+//       gA the contraction index runs over (column, sample): the reduction of
+//       the shared operand's gradient over the minibatch is the K loop.
+//   ba == bb > 1: one product per sample (grid z).
+//   ba > 1, bb == 1: per-sample products with b's stride 0; gB has a single
+//       [dj x dk] output whose K loop walks (sample, row), so the reduction
+//       over the minibatch again happens inside the kernel.
+#include "phip_internal.h"
+
+namespace phip {
+
+static int check_matmul_args(const void *a, const void *b, const void *c, uint32_t di, uint32_t dj,
+                             uint32_t dk, uint32_t ba, uint32_t bb) {
+  PHIP_REQUIRE(a != nullptr && b != nullptr && c != nullptr, "null tensor pointer");
+  PHIP_REQUIRE(di >= 1 && dj >= 1 && dk >= 1, "matrix dimensions must be positive");
+  PHIP_REQUIRE(ba >= 1 && bb >= 1 && (ba == bb || ba == 1 || bb == 1),
+               "Invalid shapes to calculate the matrix product: batch sizes %u and %u", ba, bb);
+  const uint64_t bs = ba > bb ? ba : bb;
+  const uint64_t lim = 0x7fffffffull;
+  PHIP_REQUIRE((uint64_t)dk * bs <= lim && (uint64_t)di <= lim && (uint64_t)dj <= lim,
+               "matrix dimension exceeds 2^31-1");
+  return PHIP_OK;
+}
+
+typedef int (*gemm_fn)(phip_ctx *, const Gemm &, Elem);
+
+static int gemm_dispatch(phip_ctx *ctx, const Gemm &g, Elem elem) {
+  return elem == Elem::F32 ? gemm_f32(ctx, g) : gemm_h16(ctx, g, elem);
+}
+
+static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, void *y, uint32_t di,
+                     uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  PHIP_ENTER(ctx);
+  int rc = check_matmul_args(a, b, y, di, dj, dk, ba, bb);
+  if (rc != PHIP_OK) return rc;
+  Gemm g;
+  g.A = a; g.B = b; g.C = y;
+  g.lda = di; g.ldb = dj; g.ldc = di;
+  g.a_kmajor = false;  // a(m, k) at m + k*di
+  g.b_kmajor = true;   // b(k, n) at k + n*dj
+  g.accumulate = false;
+  g.M = di; g.K = dj;
+  if (ba > 1) {
+    g.N = dk;
+    g.batch = ba;
+    g.sA = (long)di * dj;
+    g.sB = bb > 1 ? (long)dj * dk : 0;
+    g.sC = (long)di * dk;
+  } else {
+    g.N = (int)(dk * bb);
+    g.batch = 1;
+  }
+  return gemm_dispatch(ctx, g, elem);
+}
+
+static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, const void *gy, void *ga,
+                     void *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  PHIP_ENTER(ctx);
+  int rc = check_matmul_args(a, b, gy, di, dj, dk, ba, bb);
+  if (rc != PHIP_OK) return rc;
+  PHIP_REQUIRE(ga != nullptr && gb != nullptr, "null gradient pointer");
+
+  // ga[di x dj] += gy[di x dk] . b^T : A = gy (m-contiguous), B = b^T with
+  // element (k, n) at n + k*dj (n-contiguous).
+  Gemm p;
+  p.A = gy; p.B = b; p.C = ga;
+  p.lda = di; p.ldb = dj; p.ldc = di;
+  p.a_kmajor = false;
+  p.b_kmajor = false;
+  p.accumulate = true;
+  p.M = di; p.N = dj;
+  if (ba > 1) {
+    p.K = dk;
+    p.batch = ba;
+    p.sA = (long)di * dk;
+    p.sB = bb > 1 ? (long)dj * dk : 0;
+    p.sC = (long)di * dj;
+  } else {
+    p.K = (int)(dk * bb);  // contraction over (column, sample)
+    p.batch = 1;
+  }
+  rc = gemm_dispatch(ctx, p, elem);
+  if (rc != PHIP_OK) return rc;
+
+  // gb[dj x dk] += a^T . gy : A = a^T with element (m, k) at k + m*di, B = gy
+  // with element (k, n) at k + n*di (both k-contiguous).
+  Gemm q;
+  q.A = a; q.B = gy; q.C = gb;
+  q.lda = di; q.ldb = di; q.ldc = dj;
+  q.a_kmajor = true;
+  q.b_kmajor = true;
+  q.accumulate = true;
+  q.M = dj; q.K = di;
+  if (ba > 1 && bb > 1) {
+    q.N = dk;
+    q.batch = ba;
+    q.sA = (long)di * dj;
+    q.sB = (long)di * dk;
+    q.sC = (long)dj * dk;
+  } else if (ba > 1) {
+    // b is shared: one output, contraction over (sample, row).
+    q.N = dk;
+    q.batch = 1;
+    q.rbatch = ba;
+    q.rA = (long)di * dj;
+    q.rB = (long)di * dk;
+  } else {
+    q.N = (int)(dk * bb);
+    q.batch = 1;
+  }
+  return gemm_dispatch(ctx, q, elem);
+}
+
+}  // namespace phip
+
+using namespace phip;
+
+extern "C" {
+
+int phip_matmul_fw_f32(phip_ctx *ctx, const float *a, const float *b, float *y, uint32_t di, uint32_t dj,
+                       uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_fw(ctx, Elem::F32, a, b, y, di, dj, dk, ba, bb);
+}
+int phip_matmul_fw_f16(phip_ctx *ctx, const void *a, const void *b, void *y, uint32_t di, uint32_t dj,
+                       uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_fw(ctx, Elem::F16, a, b, y, di, dj, dk, ba, bb);
+}
+int phip_matmul_fw_bf16(phip_ctx *ctx, const void *a, const void *b, void *y, uint32_t di, uint32_t dj,
+                        uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_fw(ctx, Elem::BF16, a, b, y, di, dj, dk, ba, bb);
+}
+
+int phip_matmul_bw_f32(phip_ctx *ctx, const float *a, const float *b, const float *gy, float *ga,
+                       float *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_bw(ctx, Elem::F32, a, b, gy, ga, gb, di, dj, dk, ba, bb);
+}
+int phip_matmul_bw_f16(phip_ctx *ctx, const void *a, const void *b, const void *gy, void *ga, void *gb,
+                       uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_bw(ctx, Elem::F16, a, b, gy, ga, gb, di, dj, dk, ba, bb);
+}
+int phip_matmul_bw_bf16(phip_ctx *ctx, const void *a, const void *b, const void *gy, void *ga, void *gb,
+                        uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  return matmul_bw(ctx, Elem::BF16, a, b, gy, ga, gb, di, dj, dk, ba, bb);
+}
+
+}  // extern "C"

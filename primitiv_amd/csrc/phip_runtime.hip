@@ -1,0 +1,416 @@
+// Contexts, the device memory pool, copies, events and the host randomizer.
+#include <atomic>
+#include <cstring>
+#include <random>
+#include <cmath>
+#include <string>
+
+#include "phip_internal.h"
+
+namespace phip {
+
+static thread_local char g_error[1024] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Registry of live contexts, so that a handle deleter can ask whether the
+// pool it came from still exists.
+static std::mutex g_registry_mutex;
+static std::unordered_map<uint64_t, phip_ctx *> g_registry;
+static std::atomic<uint64_t> g_next_id{1};
+
+static unsigned ceil_log2(uint64_t x) {
+  unsigned s = 0;
+  while ((1ull << s) < x) ++s;
+  return s;
+}
+
+static int release_reserved_locked(phip_ctx *ctx) {
+  int rc = PHIP_OK;
+  for (auto &list : ctx->pool.reserved) {
+    while (!list.empty()) {
+      if (hipFree(list.back()) != hipSuccess) {
+        rc = fail(PHIP_ERR_RUNTIME, "hipFree failed while releasing pool blocks");
+      }
+      list.pop_back();
+    }
+  }
+  return rc;
+}
+
+static int pool_free_locked(phip_ctx *ctx, void *ptr) {
+  auto it = ctx->pool.supplied.find(ptr);
+  if (it == ctx->pool.supplied.end()) {
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "Detected to dispose unknown handle: %p", ptr);
+  }
+  ctx->pool.reserved[it->second].push_back(ptr);
+  ctx->pool.supplied.erase(it);
+  return PHIP_OK;
+}
+
+}  // namespace phip
+
+using phip::fail;
+
+extern "C" {
+
+const char *phip_last_error(void) { return phip::g_error; }
+
+int phip_device_count(int *count) {
+  PHIP_REQUIRE(count != nullptr, "null count");
+  *count = 0;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e == hipErrorNoDevice) {
+    (void)hipGetLastError();
+    return PHIP_OK;
+  }
+  PHIP_HIP(e);
+  *count = n;
+  return PHIP_OK;
+}
+
+int phip_check_support(int device_id) {
+  int n = 0;
+  int rc = phip_device_count(&n);
+  if (rc != PHIP_OK) return rc;
+  PHIP_REQUIRE(device_id >= 0 && device_id < n, "Invalid device ID: %d", device_id);
+  hipDeviceProp_t prop;
+  PHIP_HIP(hipGetDeviceProperties(&prop, device_id));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    return fail(PHIP_ERR_UNSUPPORTED,
+                "HIP device %d is %s; this backend contains gfx950 (MI355X) code only",
+                device_id, prop.gcnArchName);
+  }
+  if (prop.totalGlobalMem < (1ull << 30)) {
+    return fail(PHIP_ERR_UNSUPPORTED, "HIP device %d has less than 1 GiB of memory", device_id);
+  }
+  if (prop.warpSize != 64) {
+    return fail(PHIP_ERR_UNSUPPORTED, "HIP device %d does not run 64-wide wavefronts", device_id);
+  }
+  return PHIP_OK;
+}
+
+int phip_ctx_create(int device_id, phip_ctx **out) {
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  *out = nullptr;
+  int rc = phip_check_support(device_id);
+  if (rc != PHIP_OK) return rc;
+  PHIP_HIP(hipSetDevice(device_id));
+  phip_ctx *ctx = new phip_ctx();
+  ctx->device = device_id;
+  hipError_t e = hipGetDeviceProperties(&ctx->prop, device_id);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete ctx;
+    return fail(PHIP_ERR_RUNTIME, "context creation failed: %s", hipGetErrorString(e));
+  }
+  ctx->id = phip::g_next_id.fetch_add(1);
+  {
+    std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
+    phip::g_registry.emplace(ctx->id, ctx);
+  }
+  *out = ctx;
+  return PHIP_OK;
+}
+
+int phip_ctx_destroy(phip_ctx *ctx) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  {
+    std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
+    phip::g_registry.erase(ctx->id);
+  }
+  int rc = PHIP_OK;
+  if (hipSetDevice(ctx->device) != hipSuccess ||
+      hipStreamSynchronize(ctx->stream) != hipSuccess) {
+    rc = fail(PHIP_ERR_RUNTIME, "synchronisation failed while destroying the context");
+  }
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    // Blocks still handed out are freed too: handles may outlive the device.
+    for (auto &kv : ctx->pool.supplied) {
+      if (hipFree(kv.first) != hipSuccess) rc = fail(PHIP_ERR_RUNTIME, "hipFree failed");
+    }
+    ctx->pool.supplied.clear();
+    int r2 = phip::release_reserved_locked(ctx);
+    if (r2 != PHIP_OK) rc = r2;
+  }
+  if (hipStreamDestroy(ctx->stream) != hipSuccess) {
+    rc = fail(PHIP_ERR_RUNTIME, "hipStreamDestroy failed");
+  }
+  delete ctx;
+  return rc;
+}
+
+uint64_t phip_ctx_id(const phip_ctx *ctx) { return ctx ? ctx->id : 0; }
+
+int phip_device_info_get(phip_ctx *ctx, phip_device_info *out) {
+  PHIP_REQUIRE(ctx != nullptr && out != nullptr, "null argument");
+  std::memset(out, 0, sizeof(*out));
+  const hipDeviceProp_t &p = ctx->prop;
+  std::snprintf(out->name, sizeof(out->name), "%s", p.name);
+  std::snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+  out->device_id = ctx->device;
+  out->compute_units = p.multiProcessorCount;
+  out->clock_mhz = p.clockRate / 1000;
+  out->memory_clock_mhz = p.memoryClockRate / 1000;
+  out->memory_bus_bits = p.memoryBusWidth;
+  out->wavefront_size = p.warpSize;
+  out->lds_bytes_per_workgroup = static_cast<int32_t>(p.sharedMemPerBlock);
+  out->l2_bytes = p.l2CacheSize;
+  out->global_memory_bytes = p.totalGlobalMem;
+  return PHIP_OK;
+}
+
+int phip_describe(phip_ctx *ctx, char *buf, size_t buf_size) {
+  PHIP_REQUIRE(ctx != nullptr && buf != nullptr && buf_size > 0, "null argument");
+  const hipDeviceProp_t &p = ctx->prop;
+  std::snprintf(
+      buf, buf_size,
+      "Device %p\n"
+      "  Type: HIP\n"
+      "  Device ID: %d\n"
+      "    Name ................. %s\n"
+      "    Architecture ......... %s\n"
+      "    Global memory ........ %llu\n"
+      "    LDS per workgroup .... %zu\n"
+      "    Compute units ........ %d\n"
+      "    Wavefront size ....... %d\n"
+      "    Engine clock (kHz) ... %d\n"
+      "    Memory clock (kHz) ... %d\n"
+      "    Memory bus (bits) .... %d\n"
+      "    L2 cache ............. %d\n",
+      static_cast<void *>(ctx), ctx->device, p.name, p.gcnArchName,
+      static_cast<unsigned long long>(p.totalGlobalMem), p.sharedMemPerBlock,
+      p.multiProcessorCount, p.warpSize, p.clockRate, p.memoryClockRate,
+      p.memoryBusWidth, p.l2CacheSize);
+  return PHIP_OK;
+}
+
+int phip_sync(phip_ctx *ctx) {
+  PHIP_ENTER(ctx);
+  PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  return PHIP_OK;
+}
+
+// ---- raw memory ---------------------------------------------------------------
+
+int phip_malloc(phip_ctx *ctx, size_t bytes, void **out) {
+  PHIP_ENTER(ctx);
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  *out = nullptr;
+  if (bytes == 0) return PHIP_OK;
+  hipError_t e = hipMalloc(out, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *out = nullptr;
+    return fail(e == hipErrorOutOfMemory ? PHIP_ERR_OUT_OF_MEMORY : PHIP_ERR_RUNTIME,
+                "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+  }
+  return PHIP_OK;
+}
+
+int phip_free(phip_ctx *ctx, void *ptr) {
+  PHIP_ENTER(ctx);
+  if (ptr == nullptr) return PHIP_OK;
+  PHIP_HIP(hipFree(ptr));
+  return PHIP_OK;
+}
+
+// ---- pool ---------------------------------------------------------------------
+
+int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated) {
+  PHIP_ENTER(ctx);
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  *out = nullptr;
+  if (allocated) *allocated = 0;
+  if (bytes == 0) return PHIP_OK;
+  if (bytes < phip::Pool::kMinimumSize) bytes = phip::Pool::kMinimumSize;
+  if (bytes > (1ull << 62)) {
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "Invalid memory size: %zu", bytes);
+  }
+  const unsigned shift = phip::ceil_log2(bytes);
+  const size_t block = 1ull << shift;
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  void *ptr = nullptr;
+  auto &list = ctx->pool.reserved[shift];
+  if (!list.empty()) {
+    ptr = list.back();
+    list.pop_back();
+  } else {
+    hipError_t e = hipMalloc(&ptr, block);
+    if (e != hipSuccess) {
+      // Most likely out of memory: give back every idle block and try again.
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(ctx->stream);
+      phip::release_reserved_locked(ctx);
+      e = hipMalloc(&ptr, block);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(e == hipErrorOutOfMemory ? PHIP_ERR_OUT_OF_MEMORY : PHIP_ERR_RUNTIME,
+                  "Memory allocation failed. Requested size: %zu (%s)", block,
+                  hipGetErrorString(e));
+    }
+  }
+  ctx->pool.supplied.emplace(ptr, shift);
+  *out = ptr;
+  if (allocated) *allocated = block;
+  return PHIP_OK;
+}
+
+int phip_pool_free(phip_ctx *ctx, void *ptr) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  if (ptr == nullptr) return PHIP_OK;
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  return phip::pool_free_locked(ctx, ptr);
+}
+
+int phip_pool_free_by_id(uint64_t ctx_id, void *ptr) {
+  if (ptr == nullptr) return PHIP_OK;
+  std::lock_guard<std::mutex> reg(phip::g_registry_mutex);
+  auto it = phip::g_registry.find(ctx_id);
+  if (it == phip::g_registry.end()) return PHIP_OK;  // pool already gone
+  std::lock_guard<std::mutex> lock(it->second->mutex);
+  return phip::pool_free_locked(it->second, ptr);
+}
+
+int phip_pool_release_reserved(phip_ctx *ctx) {
+  PHIP_ENTER(ctx);
+  // Idle blocks may still be read by kernels enqueued before they were freed.
+  PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  return phip::release_reserved_locked(ctx);
+}
+
+int phip_pool_stats(phip_ctx *ctx, uint64_t *supplied_bytes, uint64_t *reserved_bytes) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  uint64_t s = 0, r = 0;
+  for (auto &kv : ctx->pool.supplied) s += 1ull << kv.second;
+  for (size_t i = 0; i < ctx->pool.reserved.size(); ++i) {
+    r += (1ull << i) * ctx->pool.reserved[i].size();
+  }
+  if (supplied_bytes) *supplied_bytes = s;
+  if (reserved_bytes) *reserved_bytes = r;
+  return PHIP_OK;
+}
+
+// ---- copies -------------------------------------------------------------------
+
+int phip_memcpy_h2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  PHIP_ENTER(ctx);
+  if (bytes == 0) return PHIP_OK;
+  PHIP_REQUIRE(dst != nullptr && src != nullptr, "null pointer in h2d copy");
+  PHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  return PHIP_OK;
+}
+
+int phip_memcpy_d2h(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  PHIP_ENTER(ctx);
+  if (bytes == 0) return PHIP_OK;
+  PHIP_REQUIRE(dst != nullptr && src != nullptr, "null pointer in d2h copy");
+  PHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  return PHIP_OK;
+}
+
+int phip_memcpy_d2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  PHIP_ENTER(ctx);
+  if (bytes == 0) return PHIP_OK;
+  PHIP_REQUIRE(dst != nullptr && src != nullptr, "null pointer in d2d copy");
+  PHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return PHIP_OK;
+}
+
+// ---- events -------------------------------------------------------------------
+
+int phip_event_create(phip_ctx *ctx, phip_event **out) {
+  PHIP_ENTER(ctx);
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  phip_event *ev = new phip_event();
+  ev->device = ctx->device;
+  hipError_t e = hipEventCreate(&ev->ev);
+  if (e != hipSuccess) {
+    delete ev;
+    return fail(PHIP_ERR_RUNTIME, "hipEventCreate failed: %s", hipGetErrorString(e));
+  }
+  *out = ev;
+  return PHIP_OK;
+}
+
+int phip_event_destroy(phip_event *ev) {
+  if (ev == nullptr) return PHIP_OK;
+  hipError_t e = hipEventDestroy(ev->ev);
+  delete ev;
+  if (e != hipSuccess) return fail(PHIP_ERR_RUNTIME, "hipEventDestroy failed");
+  return PHIP_OK;
+}
+
+int phip_event_record(phip_ctx *ctx, phip_event *ev) {
+  PHIP_ENTER(ctx);
+  PHIP_REQUIRE(ev != nullptr, "null event");
+  PHIP_HIP(hipEventRecord(ev->ev, ctx->stream));
+  return PHIP_OK;
+}
+
+int phip_event_elapsed_ms(phip_event *start, phip_event *stop, float *ms) {
+  PHIP_REQUIRE(start && stop && ms, "null argument");
+  PHIP_HIP(hipEventSynchronize(stop->ev));
+  PHIP_HIP(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return PHIP_OK;
+}
+
+}  // extern "C"
+
+// ---- host randomizer ------------------------------------------------------------
+
+struct phip_randomizer {
+  std::mt19937 rng;
+  explicit phip_randomizer(uint32_t seed) : rng(seed) {}
+};
+
+extern "C" {
+
+int phip_randomizer_create(uint32_t seed, phip_randomizer **out) {
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  *out = new phip_randomizer(seed);
+  return PHIP_OK;
+}
+
+int phip_randomizer_destroy(phip_randomizer *r) {
+  delete r;
+  return PHIP_OK;
+}
+
+int phip_randomizer_fill_uniform(phip_randomizer *r, float lower, float upper, size_t n,
+                                 float *host_out) {
+  PHIP_REQUIRE(r != nullptr && (host_out != nullptr || n == 0), "null argument");
+  PHIP_REQUIRE(lower < upper, "uniform bounds must satisfy lower < upper");
+  // One distribution object per fill; the open end is the lower one.
+  std::uniform_real_distribution<float> dist(lower, upper);
+  const float lower_eps = std::nextafter(lower, upper);
+  for (size_t i = 0; i < n; ++i) {
+    const float x = dist(r->rng);
+    host_out[i] = x < lower_eps ? upper : x;
+  }
+  return PHIP_OK;
+}
+
+int phip_randomizer_fill_normal(phip_randomizer *r, float mean, float sd, size_t n,
+                                float *host_out) {
+  PHIP_REQUIRE(r != nullptr && (host_out != nullptr || n == 0), "null argument");
+  PHIP_REQUIRE(sd > 0.0f, "standard deviation must be positive");
+  std::normal_distribution<float> dist(mean, sd);
+  for (size_t i = 0; i < n; ++i) host_out[i] = dist(r->rng);
+  return PHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,426 @@
+"""Python mirror of primitiv's Device front for the matmul path.
+
+This is the thin host side used by the tests and the benchmark: the same
+method names, argument meaning and error behaviour as the reference's
+`Device`, `Tensor` and `Shape` (primitiv/core/device.{h,cc},
+primitiv/core/tensor.{h,cc}, primitiv/core/shape.{h,cc}), restricted to what
+the matmul path touches.  All arithmetic happens in libphip.so on the GPU; this
+file only checks shapes, owns handles and moves bytes.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import Error
+
+
+class Shape:
+    """Up to 8 dimensions plus a minibatch size (primitiv/core/shape.h).
+
+    Trailing dimensions of size 1 are not stored; `shape[i]` past the depth
+    reads 1 (shape.h:55).
+    """
+
+    MAX_DEPTH = 8
+
+    def __init__(self, dims=(), batch=1):
+        dims = [int(d) for d in dims]
+        if len(dims) > self.MAX_DEPTH:
+            raise Error("Exceeds dimension depth limit at Shape.init: %d > %d" % (len(dims), self.MAX_DEPTH))
+        while dims and dims[-1] == 1:
+            dims.pop()
+        if any(d <= 0 for d in dims) or batch <= 0:
+            raise Error("Invalid shape: %s x %d" % (dims, batch))
+        self._dims = tuple(dims)
+        self._batch = int(batch)
+        vol = 1
+        for d in dims:
+            vol *= d
+        self._volume = vol
+
+    def __getitem__(self, i):
+        return self._dims[i] if i < len(self._dims) else 1
+
+    def dims(self):
+        return list(self._dims)
+
+    def depth(self):
+        return len(self._dims)
+
+    def batch(self):
+        return self._batch
+
+    def volume(self):
+        return self._volume
+
+    def size(self):
+        return self._batch * self._volume
+
+    def has_batch(self):
+        return self._batch > 1
+
+    def has_compatible_batch(self, rhs):
+        return self._batch == rhs._batch or self._batch == 1 or rhs._batch == 1
+
+    def is_matrix(self):
+        return len(self._dims) <= 2
+
+    def has_same_dims(self, rhs):
+        return self._dims == rhs._dims
+
+    def resize_batch(self, batch):
+        return Shape(self._dims, batch)
+
+    def to_string(self):
+        return "[%s]x%d" % (",".join(str(d) for d in self._dims), self._batch)
+
+    __repr__ = to_string
+
+    def __eq__(self, rhs):
+        return isinstance(rhs, Shape) and self._dims == rhs._dims and self._batch == rhs._batch
+
+    def __ne__(self, rhs):
+        return not self.__eq__(rhs)
+
+    def __hash__(self):
+        return hash((self._dims, self._batch))
+
+
+def _as_shape(s):
+    return s if isinstance(s, Shape) else Shape(s)
+
+
+class shape_ops:
+    """Result-shape rules (primitiv/core/shape_ops.cc)."""
+
+    @staticmethod
+    def matmul(l, r):
+        # shape_ops.cc:152-160
+        if (not l.is_matrix() or not r.is_matrix() or l[1] != r[0]
+                or not l.has_compatible_batch(r)):
+            raise Error("Invalid shapes to calculate the matrix product: %s, %s"
+                        % (l.to_string(), r.to_string()))
+        return Shape([l[0], r[1]], max(l.batch(), r.batch()))
+
+    @staticmethod
+    def batch_sum(x):
+        return x.resize_batch(1)
+
+
+class _Handle:
+    """One pool block; returned to the pool of its context when dropped,
+    silently if that context is already gone (primitiv/core/memory_pool.h:22-35)."""
+
+    __slots__ = ("ptr", "ctx_id", "allocated", "sharers")
+
+    def __init__(self, ptr, ctx_id, allocated):
+        self.ptr, self.ctx_id, self.allocated = ptr, ctx_id, allocated
+        self.sharers = 0  # tensors that currently refer to this block
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                _lib.lib().phip_pool_free_by_id(self.ctx_id, self.ptr)
+        except Exception:
+            pass
+
+
+class Tensor:
+    """Value handle with copy-on-write sharing (primitiv/core/tensor.{h,cc})."""
+
+    def __init__(self, shape=None, device=None, handle=None):
+        self._shape = shape
+        self._device = device
+        self._handle = handle
+        if handle is not None:
+            handle.sharers += 1
+
+    def __del__(self):
+        if getattr(self, "_handle", None) is not None:
+            self._handle.sharers -= 1
+
+    def valid(self):
+        return self._handle is not None
+
+    def _check_valid(self):
+        if not self.valid():
+            raise Error("Invalid tensor.")
+
+    def shape(self):
+        self._check_valid()
+        return self._shape
+
+    def device(self):
+        self._check_valid()
+        return self._device
+
+    def allocated_size(self):
+        self._check_valid()
+        return self._handle.allocated
+
+    def handle(self):
+        self._check_valid()
+        return self._handle.ptr
+
+    def mutable_handle(self):
+        """Raw pointer for writing; clones the block first when it is shared
+        (tensor.cc:33-41)."""
+        self._check_valid()
+        if self._handle.sharers > 1:
+            clone = self._device.copy_tensor(self)
+            self._handle.sharers -= 1
+            self._handle = clone._handle
+            self._handle.sharers += 1
+        return self._handle.ptr
+
+    def copy(self):
+        """Copy construction: shares the handle until one side is written."""
+        return Tensor(self._shape, self._device, self._handle)
+
+    def to_vector(self):
+        self._check_valid()
+        return self._device.tensor_to_vector(self)
+
+    def to_float(self):
+        self._check_valid()
+        if self._shape.size() != 1:
+            raise Error("Tensor has more than 1 values. shape = " + self._shape.to_string())
+        return float(self.to_vector()[0])
+
+    def inplace_add(self, x):
+        self._check_valid()
+        self._device.inplace_add(x, self)
+        return self
+
+    __iadd__ = inplace_add
+
+
+class DeviceType:
+    # the reference's enum (primitiv/core/device.h:17-35) extended by one group
+    GROUP_HIP = 0x00030000
+    HIP = 0x00030000
+    HIP16 = 0x00030001
+
+
+class HIP:
+    """fp32 device (mirrors primitiv::devices::CUDA's public face,
+    primitiv/devices/cuda/device.h:27-62, for the calls on the matmul path)."""
+
+    _SUFFIX = "f32"
+    _ITEMSIZE = 4
+
+    @staticmethod
+    def num_devices():
+        n = ctypes.c_int(0)
+        _lib.call("phip_device_count", ctypes.byref(n))
+        return n.value
+
+    @staticmethod
+    def assert_support(device_id):
+        _lib.call("phip_check_support", int(device_id))
+
+    @staticmethod
+    def check_support(device_id):
+        try:
+            HIP.assert_support(device_id)
+        except Error:
+            return False
+        return True
+
+    def __init__(self, device_id, rng_seed=None):
+        if device_id < 0:
+            raise Error("Invalid device ID: %d" % device_id)
+        self._ctx = ctypes.c_void_p()
+        _lib.call("phip_ctx_create", int(device_id), ctypes.byref(self._ctx))
+        self._ctx_id = _lib.lib().phip_ctx_id(self._ctx)
+        self._device_id = int(device_id)
+        self._rng_seed = rng_seed
+
+    def close(self):
+        if self._ctx:
+            ctx, self._ctx = self._ctx, None
+            _lib.call("phip_ctx_destroy", ctx)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- identity ---------------------------------------------------------
+    def type(self):
+        return DeviceType.HIP
+
+    def ctx(self):
+        return self._ctx
+
+    def info(self):
+        out = _lib.DeviceInfo()
+        _lib.call("phip_device_info_get", self._ctx, ctypes.byref(out))
+        return out
+
+    def dump_description(self):
+        buf = ctypes.create_string_buffer(2048)
+        _lib.call("phip_describe", self._ctx, buf, len(buf))
+        return buf.value.decode()
+
+    def sync(self):
+        _lib.call("phip_sync", self._ctx)
+
+    # -- storage ----------------------------------------------------------
+    def _elements_to_bytes(self, n):
+        return self._ITEMSIZE * n
+
+    def new_raw_tensor(self, shape):
+        # device.cc:20-24 -> new_handle (devices/cuda/ops/new_handle.cu:10-12)
+        shape = _as_shape(shape)
+        ptr = ctypes.c_void_p()
+        allocated = ctypes.c_size_t(0)
+        _lib.call("phip_pool_alloc", self._ctx, self._elements_to_bytes(shape.size()),
+                  ctypes.byref(ptr), ctypes.byref(allocated))
+        return Tensor(shape, self, _Handle(ptr.value, self._ctx_id, allocated.value))
+
+    def _check_device(self, x):
+        # device.cc:11-16
+        if x.device() is not self:
+            raise Error("Device mismatched.")
+
+    def _upload(self, ptr, host):
+        _lib.call("phip_memcpy_h2d", self._ctx, ptr, host.ctypes.data, host.nbytes)
+
+    def _download(self, ptr, n):
+        out = np.empty(n, dtype=np.float32)
+        _lib.call("phip_memcpy_d2h", self._ctx, out.ctypes.data, ptr, out.nbytes)
+        return out
+
+    def new_tensor_by_constant(self, shape, k):
+        ret = self.new_raw_tensor(shape)
+        self.reset_tensor(k, ret)
+        return ret
+
+    def new_tensor_by_array(self, shape, values):
+        ret = self.new_raw_tensor(shape)
+        self.reset_tensor_by_array(values, ret)
+        return ret
+
+    def new_tensor_by_vector(self, shape, values):
+        # device.cc:42-49
+        shape = _as_shape(shape)
+        values = np.ascontiguousarray(np.asarray(values, dtype=np.float32).reshape(-1))
+        if values.size != shape.size():
+            raise Error("Data sizes mismatched. required: %d (%s) != actual: %d"
+                        % (shape.size(), shape.to_string(), values.size))
+        return self.new_tensor_by_array(shape, values)
+
+    def reset_tensor(self, k, x):
+        self._check_device(x)
+        _lib.call("phip_fill_" + self._SUFFIX, self._ctx, x.mutable_handle(), float(k), x.shape().size())
+
+    def reset_tensor_by_array(self, values, x):
+        self._check_device(x)
+        values = np.ascontiguousarray(np.asarray(values, dtype=np.float32).reshape(-1))
+        n = x.shape().size()
+        if values.size < n:
+            raise Error("host array is shorter than the tensor")
+        self._upload(x.mutable_handle(), values[:n])
+
+    def tensor_to_vector(self, x):
+        self._check_device(x)
+        return self._download(x.handle(), x.shape().size())
+
+    def copy_tensor(self, x):
+        # devices/cuda/ops/copy_tensor.cu:10-30: same device type -> D2D,
+        # anything else bounces through the host.
+        ret = self.new_raw_tensor(x.shape())
+        if isinstance(x.device(), HIP) and x.device().type() == self.type():
+            _lib.call("phip_memcpy_d2d", self._ctx, ret._handle.ptr, x.handle(),
+                      self._elements_to_bytes(x.shape().size()))
+        else:
+            self.reset_tensor_by_array(x.to_vector(), ret)
+        return ret
+
+    # -- the matmul path --------------------------------------------------
+    def matmul_fw(self, a, b):
+        # DEV_FW_AB, device.cc:268-275,418
+        self._check_device(a)
+        self._check_device(b)
+        y = self.new_raw_tensor(shape_ops.matmul(a.shape(), b.shape()))
+        sa, sb = a.shape(), b.shape()
+        _lib.call("phip_matmul_fw_" + self._SUFFIX, self._ctx, a.handle(), b.handle(),
+                  y.mutable_handle(), sa[0], sa[1], sb[1], sa.batch(), sb.batch())
+        return y
+
+    def matmul_bw(self, a, b, y, gy, ga, gb):
+        # DEV_BW_AB, device.cc:277-301,453
+        for t in (a, b, y, gy, ga, gb):
+            self._check_device(t)
+        if (a.shape() != ga.shape() or b.shape() != gb.shape() or y.shape() != gy.shape()
+                or y.shape() != shape_ops.matmul(a.shape(), b.shape())):
+            raise Error("Shape mismatched at matmul_bw. a: %s, b: %s, y: %s, gy: %s, ga: %s, gb: %s"
+                        % tuple(t.shape().to_string() for t in (a, b, y, gy, ga, gb)))
+        sa, sb = a.shape(), b.shape()
+        # writable pointers first: taking them may clone a shared block
+        pga, pgb = ga.mutable_handle(), gb.mutable_handle()
+        _lib.call("phip_matmul_bw_" + self._SUFFIX, self._ctx, a.handle(), b.handle(),
+                  gy.handle(), pga, pgb, sa[0], sa[1], sb[1], sa.batch(), sb.batch())
+
+    def inplace_add(self, x, y):
+        # device.cc:692-703
+        self._check_device(x)
+        self._check_device(y)
+        sx, sy = x.shape(), y.shape()
+        if not sx.has_same_dims(sy) or not sx.has_compatible_batch(sy):
+            raise Error("Attempted to add values of shape %s to shape %s"
+                        % (sx.to_string(), sy.to_string()))
+        _lib.call("phip_inplace_add_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(),
+                  sy.volume(), sx.batch(), sy.batch())
+        return y
+
+    def batch_sum_fw(self, x):
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.batch_sum(x.shape()))
+        _lib.call("phip_batch_sum_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(),
+                  x.shape().volume(), x.shape().batch())
+        return y
+
+
+class HIP16(HIP):
+    """Half-storage device: 16-bit tensors on the GPU, float at the API edge,
+    fp32 accumulation (the counterpart of primitiv::devices::CUDA16,
+    primitiv/devices/cuda16/).  `storage` is "f16" or "bf16"."""
+
+    _ITEMSIZE = 2
+
+    def __init__(self, device_id, rng_seed=None, storage="f16"):
+        if storage not in ("f16", "bf16"):
+            raise Error("unknown storage type: %r" % (storage,))
+        super().__init__(device_id, rng_seed)
+        self._SUFFIX = storage
+
+    def type(self):
+        return DeviceType.HIP16
+
+    def _elements_to_bytes(self, n):
+        # element count rounded up to even (devices/cuda16/ops/new_handle.cu:10-16)
+        return 2 * (n + (n & 1))
+
+    def _staging(self, n):
+        ptr = ctypes.c_void_p()
+        _lib.call("phip_pool_alloc", self._ctx, 4 * n, ctypes.byref(ptr), None)
+        return _Handle(ptr.value, self._ctx_id, 0)
+
+    def _upload(self, ptr, host):
+        # host floats -> pooled fp32 staging block -> 16-bit storage
+        # (devices/cuda16/ops/reset_tensor_by_array.cu:19-30)
+        tmp = self._staging(host.size)
+        _lib.call("phip_memcpy_h2d", self._ctx, tmp.ptr, host.ctypes.data, host.nbytes)
+        _lib.call("phip_cvt_f32_to_" + self._SUFFIX, self._ctx, tmp.ptr, ptr, host.size)
+
+    def _download(self, ptr, n):
+        # (devices/cuda16/ops/tensor_to_vector.cu:19-32)
+        tmp = self._staging(n)
+        _lib.call("phip_cvt_%s_to_f32" % self._SUFFIX, self._ctx, ptr, tmp.ptr, n)
+        out = np.empty(n, dtype=np.float32)
+        _lib.call("phip_memcpy_d2h", self._ctx, out.ctypes.data, tmp.ptr, out.nbytes)
+        return out

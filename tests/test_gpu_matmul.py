@@ -1,0 +1,319 @@
+"""Parity of the HIP matmul path with the CPU oracle, through the C ABI.
+
+Tolerance gate (stated with every check): max|x - ref| / max|ref| per output
+tensor; fp32 device <= 1e-4, 16-bit storage <= 2e-2 against the fp32 oracle
+fed the un-rounded inputs.  Integer-valued golden vectors of the reference's
+own tests must match to 4 ULPs as they do there.
+"""
+import numpy as np
+import pytest
+
+import oracle
+import primitiv_amd as pa
+from primitiv_amd.configs import WORKLOADS
+from util import norm_rel_err, np_matmul_bw, np_matmul_fw, vector_match
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-4
+H16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = pa.HIP(0)
+    yield d
+    d.close()
+
+
+@pytest.fixture(scope="module")
+def dev16():
+    d = pa.HIP16(0, storage="f16")
+    yield d
+    d.close()
+
+
+@pytest.fixture(scope="module")
+def devbf16():
+    d = pa.HIP16(0, storage="bf16")
+    yield d
+    d.close()
+
+
+def _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb):
+    bs = max(ba, bb)
+    ta = dev.new_tensor_by_vector(pa.Shape([di, dj], ba), a)
+    tb = dev.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    ty = dev.matmul_fw(ta, tb)
+    assert ty.shape() == pa.Shape([di, dk], bs)
+    tgy = dev.new_tensor_by_vector(ty.shape(), gy)
+    tga = dev.new_tensor_by_vector(ta.shape(), ga0)
+    tgb = dev.new_tensor_by_vector(tb.shape(), gb0)
+    dev.matmul_bw(ta, tb, ty, tgy, tga, tgb)
+    return ty.to_vector(), tga.to_vector(), tgb.to_vector()
+
+
+# ---- the reference's golden vectors -----------------------------------------
+
+def test_golden_forward(dev, golden):
+    for c in golden["matmul_fw"]:
+        a = dev.new_tensor_by_vector(pa.Shape([c["di"], c["dj"]], c["ba"]), c["a"])
+        b = dev.new_tensor_by_vector(pa.Shape([c["dj"], c["dk"]], c["bb"]), c["b"])
+        y = dev.matmul_fw(a, b)
+        assert y.shape() == pa.Shape([c["di"], c["dk"]], max(c["ba"], c["bb"]))
+        assert vector_match(c["y"], y.to_vector()), c["source"]
+
+
+def test_golden_forward_large(dev, golden):
+    n = golden["matmul_fw_large"]["n"]
+    i = np.arange(n, dtype=np.float64)
+    a_data = np.tile(i / 16.0, n)
+    b_data = np.repeat(i / 16.0, n)
+    y1 = np.outer(i, i).T.reshape(-1) * n / 256.0
+    y2 = np.full(n * n, np.sum(i * i) / 256.0)
+    a = dev.new_tensor_by_vector([n, n], a_data)
+    b = dev.new_tensor_by_vector([n, n], b_data)
+    assert vector_match(y1, dev.matmul_fw(a, b).to_vector())
+    assert vector_match(y2, dev.matmul_fw(b, a).to_vector())
+
+
+def test_golden_backward(dev, golden):
+    for c in golden["matmul_bw"] + [golden["matmul_operator"]]:
+        a = dev.new_tensor_by_vector(pa.Shape([c["di"], c["dj"]], c["ba"]), c["a"])
+        b = dev.new_tensor_by_vector(pa.Shape([c["dj"], c["dk"]], c["bb"]), c["b"])
+        y = dev.matmul_fw(a, b)
+        gy = dev.new_tensor_by_vector(y.shape(), c["gy"])
+        ga = dev.new_tensor_by_constant(a.shape(), 0)
+        gb = dev.new_tensor_by_constant(b.shape(), 0)
+        dev.matmul_bw(a, b, y, gy, ga, gb)
+        assert vector_match(c["ga"], ga.to_vector()), c["source"]
+        assert vector_match(c["gb"], gb.to_vector()), c["source"]
+
+
+def test_invalid_matmul(dev, golden):
+    # test/tensor_forward_test.cc:1907-1927
+    for c in golden["shape_matmul_invalid"]["cases"]:
+        a = dev.new_tensor_by_constant(pa.Shape(c["a"], c["ba"]), 0)
+        b = dev.new_tensor_by_constant(pa.Shape(c["b"], c["bb"]), 0)
+        with pytest.raises(pa.Error):
+            dev.matmul_fw(a, b)
+
+
+def test_golden_half_storage(dev16, devbf16, golden):
+    # small integers are exact in either 16-bit format; the reference's own
+    # half device needs 16384 ULPs on CheckMatMulAB (tensor_forward_test.cc:1838-1842)
+    for d in (dev16, devbf16):
+        for c in golden["matmul_fw"]:
+            a = d.new_tensor_by_vector(pa.Shape([c["di"], c["dj"]], c["ba"]), c["a"])
+            b = d.new_tensor_by_vector(pa.Shape([c["dj"], c["dk"]], c["bb"]), c["b"])
+            y = d.matmul_fw(a, b).to_vector()
+            assert norm_rel_err(y, c["y"]) <= (2.0 ** -9 if d is dev16 else 2.0 ** -8), c["source"]
+        for c in golden["matmul_bw"] + [golden["matmul_operator"]]:
+            a = d.new_tensor_by_vector(pa.Shape([c["di"], c["dj"]], c["ba"]), c["a"])
+            b = d.new_tensor_by_vector(pa.Shape([c["dj"], c["dk"]], c["bb"]), c["b"])
+            y = d.matmul_fw(a, b)
+            gy = d.new_tensor_by_vector(y.shape(), c["gy"])
+            ga = d.new_tensor_by_constant(a.shape(), 0)
+            gb = d.new_tensor_by_constant(b.shape(), 0)
+            d.matmul_bw(a, b, y, gy, ga, gb)
+            assert vector_match(c["ga"], ga.to_vector()), c["source"]
+            assert vector_match(c["gb"], gb.to_vector()), c["source"]
+
+
+# ---- random shapes against the oracle ------------------------------------------
+
+SHAPES = [  # di, dj, dk : aligned, ragged, degenerate, larger than one tile in every direction
+    (1, 1, 1), (1, 5, 1), (7, 1, 3), (2, 3, 4), (33, 17, 65), (64, 64, 64),
+    (123, 123, 123), (128, 128, 128), (130, 70, 258), (257, 129, 31), (300, 20, 5),
+    (8, 1000, 8), (5, 4097, 3), (650, 64, 1), (512, 96, 260),
+]
+BATCHES = [(1, 1), (3, 3), (1, 3), (3, 1), (1, 37), (37, 1)]
+
+
+@pytest.mark.parametrize("ba,bb", BATCHES)
+def test_random_shapes_f32(dev, ba, bb):
+    rng = np.random.default_rng(100 * ba + bb)
+    for di, dj, dk in SHAPES:
+        bs = max(ba, bb)
+        if di * dj * dk * bs > 40_000_000:
+            continue
+        a = rng.standard_normal(di * dj * ba).astype(np.float32)
+        b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+        gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+        ga0 = rng.standard_normal(a.size).astype(np.float32)
+        gb0 = rng.standard_normal(b.size).astype(np.float32)
+        y, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+        ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 4)
+        rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 4)
+        tag = "shape (%d,%d,%d) batch (%d,%d)" % (di, dj, dk, ba, bb)
+        assert norm_rel_err(y, ry) <= F32_TOL, "y " + tag
+        assert norm_rel_err(ga, rga) <= F32_TOL, "ga " + tag
+        assert norm_rel_err(gb, rgb) <= F32_TOL, "gb " + tag
+
+
+@pytest.mark.parametrize("which", ["f16", "bf16"])
+@pytest.mark.parametrize("ba,bb", [(1, 1), (3, 3), (1, 5), (5, 1)])
+def test_random_shapes_h16(dev16, devbf16, which, ba, bb):
+    d = dev16 if which == "f16" else devbf16
+    tol = H16_TOL
+    rng = np.random.default_rng(7 * ba + bb)
+    for di, dj, dk in SHAPES:
+        bs = max(ba, bb)
+        a = rng.standard_normal(di * dj * ba).astype(np.float32)
+        b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+        gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+        ga0 = rng.standard_normal(a.size).astype(np.float32)
+        gb0 = rng.standard_normal(b.size).astype(np.float32)
+        y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+        ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 4)
+        rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 4)
+        tag = "%s shape (%d,%d,%d) batch (%d,%d)" % (which, di, dj, dk, ba, bb)
+        assert norm_rel_err(y, ry) <= tol, "y " + tag
+        assert norm_rel_err(ga, rga) <= tol, "ga " + tag
+        assert norm_rel_err(gb, rgb) <= tol, "gb " + tag
+
+
+def test_f16_matches_oracle_on_rounded_inputs(dev16):
+    # With inputs already representable in fp16 the only error left is the
+    # final rounding of the output (<= 2^-11 relative per element) on top of
+    # fp32 accumulation: a far tighter gate than 2e-2.
+    rng = np.random.default_rng(5)
+    di, dj, dk, ba, bb = 200, 160, 72, 1, 3
+    r16 = lambda x: x.astype(np.float16).astype(np.float32)
+    a = r16(rng.standard_normal(di * dj * ba).astype(np.float32))
+    b = r16(rng.standard_normal(dj * dk * bb).astype(np.float32))
+    gy = r16(rng.standard_normal(di * dk * bb).astype(np.float32))
+    z = lambda n: np.zeros(n, dtype=np.float32)
+    y, ga, gb = _fw_bw(dev16, a, b, gy, z(a.size), z(b.size), di, dj, dk, ba, bb)
+    ry = np_matmul_fw(a, b, di, dj, dk, ba, bb)
+    rga, rgb = np_matmul_bw(a, b, gy, di, dj, dk, ba, bb)
+    for got, ref in ((y, ry), (ga, rga), (gb, rgb)):
+        ref16 = ref.astype(np.float16).astype(np.float64)
+        # allow one fp16 ULP of the largest magnitude for accumulation-order ties
+        assert np.max(np.abs(got - ref16)) <= np.max(np.abs(ref)) * 2.0 ** -10
+
+
+# ---- properties that hold at any size ------------------------------------------
+
+def test_backward_accumulates_and_forward_overwrites(dev):
+    rng = np.random.default_rng(11)
+    di, dj, dk, ba, bb = 96, 80, 48, 1, 4
+    a = rng.standard_normal(di * dj).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bb).astype(np.float32)
+    ta = dev.new_tensor_by_vector(pa.Shape([di, dj]), a)
+    tb = dev.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    ty = dev.matmul_fw(ta, tb)
+    tgy = dev.new_tensor_by_vector(ty.shape(), gy)
+    ga = dev.new_tensor_by_constant(ta.shape(), 0)
+    gb = dev.new_tensor_by_constant(tb.shape(), 0)
+    dev.matmul_bw(ta, tb, ty, tgy, ga, gb)
+    ga1, gb1 = ga.to_vector(), gb.to_vector()
+    dev.matmul_bw(ta, tb, ty, tgy, ga, gb)
+    assert norm_rel_err(ga.to_vector(), 2 * ga1) <= 1e-6
+    assert norm_rel_err(gb.to_vector(), 2 * gb1) <= 1e-6
+    # forward into a block that held other data gives the same result
+    y1 = ty.to_vector()
+    del ty
+    junk = dev.new_tensor_by_constant(pa.Shape([di, dk], bb), 123.0)
+    del junk
+    assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), y1)
+
+
+def test_copy_on_write_gradient(dev):
+    # a gradient tensor that shares its block must be cloned before the
+    # backward pass adds into it (primitiv/core/tensor.cc:33-41)
+    a = dev.new_tensor_by_vector([2, 2], [1, 2, 3, 4])
+    b = dev.new_tensor_by_vector([2, 2], [1, 0, 0, 2])
+    y = dev.matmul_fw(a, b)
+    gy = dev.new_tensor_by_vector([2, 2], [1, -1, 2, -2])
+    ga = dev.new_tensor_by_constant([2, 2], 0)
+    gb = dev.new_tensor_by_constant([2, 2], 0)
+    shared = ga.copy()
+    dev.matmul_bw(a, b, y, gy, ga, gb)
+    assert vector_match([1, -1, 4, -4], ga.to_vector())
+    assert vector_match([0, 0, 0, 0], shared.to_vector())
+
+
+def test_broadcast_equals_tiled(dev):
+    rng = np.random.default_rng(13)
+    di, dj, dk, n = 70, 50, 30, 6
+    a = rng.standard_normal(di * dj).astype(np.float32)
+    b = rng.standard_normal(dj * dk * n).astype(np.float32)
+    gy = rng.standard_normal(di * dk * n).astype(np.float32)
+    z = lambda m: np.zeros(m, dtype=np.float32)
+    y1, ga1, gb1 = _fw_bw(dev, a, b, gy, z(a.size), z(b.size), di, dj, dk, 1, n)
+    at = np.tile(a, n)
+    yn, gan, gbn = _fw_bw(dev, at, b, gy, z(at.size), z(b.size), di, dj, dk, n, n)
+    assert norm_rel_err(y1, yn) <= 1e-6
+    assert norm_rel_err(gb1, gbn) <= 1e-6
+    assert norm_rel_err(ga1, gan.reshape(n, -1).sum(0)) <= 1e-5
+
+
+# ---- the benchmark workloads at full size --------------------------------------
+
+def _run_workload(dev, w, steps):
+    a, bs, gys = w.inputs(seed=0, steps=steps)
+    ta = dev.new_tensor_by_vector(pa.Shape([w.di, w.dj], w.ba), a)
+    ga = dev.new_tensor_by_constant(ta.shape(), 0)
+    outs = []
+    for t in range(steps):
+        tb = dev.new_tensor_by_vector(pa.Shape([w.dj, w.dk], w.bb), bs[t])
+        ty = dev.matmul_fw(ta, tb)
+        tgy = dev.new_tensor_by_vector(ty.shape(), gys[t])
+        gb = dev.new_tensor_by_constant(tb.shape(), 0)
+        dev.matmul_bw(ta, tb, ty, tgy, ga, gb)   # ga persists across steps
+        outs.append((ty.to_vector(), gb.to_vector()))
+    return a, bs, gys, outs, ga.to_vector()
+
+
+@pytest.mark.parametrize("name,steps", [("dense", 1), ("rnn_gate", 30), ("square_batched", 1),
+                                        ("output_projection", 5)])
+def test_workload_f32(dev, name, steps):
+    w = WORKLOADS[name]
+    a, bs, gys, outs, ga = _run_workload(dev, w, steps)
+    rga = np.zeros(a.size, dtype=np.float32)
+    for t in range(steps):
+        ry = oracle.matmul_fw(a, bs[t], w.di, w.dj, w.dk, w.ba, w.bb, 8)
+        rga, rgb = oracle.matmul_bw(a, bs[t], gys[t], rga, np.zeros(bs[t].size, np.float32),
+                                    w.di, w.dj, w.dk, w.ba, w.bb, 8)
+        assert norm_rel_err(outs[t][0], ry) <= w.tolerance, "%s step %d y" % (name, t)
+        assert norm_rel_err(outs[t][1], rgb) <= w.tolerance, "%s step %d gb" % (name, t)
+    assert norm_rel_err(ga, rga) <= w.tolerance, name + " ga"
+
+
+def test_workload_half_storage_sampled(dev16):
+    # Full size on the GPU; the oracle recomputes sampled rows / columns of each
+    # output from the un-rounded fp32 inputs (any row block of y depends only on
+    # the same rows of a, and so on), which it finishes in seconds.
+    w = WORKLOADS["half_storage"]
+    a, bs, gys = w.inputs(seed=0)
+    b, gy = bs[0], gys[0]
+    di, dj, dk, n = w.di, w.dj, w.dk, w.bb
+    ta = dev16.new_tensor_by_vector(pa.Shape([di, dj]), a)
+    tb = dev16.new_tensor_by_vector(pa.Shape([dj, dk], n), b)
+    ty = dev16.matmul_fw(ta, tb)
+    tgy = dev16.new_tensor_by_vector(ty.shape(), gy)
+    ga = dev16.new_tensor_by_constant(ta.shape(), 0)
+    gb = dev16.new_tensor_by_constant(tb.shape(), 0)
+    dev16.matmul_bw(ta, tb, ty, tgy, ga, gb)
+    y = ty.to_vector().reshape(n * dk, di)        # [column of Y'][row]
+    gav = ga.to_vector().reshape(dj, di)
+    gbv = gb.to_vector().reshape(n * dk, dj)
+    rng = np.random.default_rng(0)
+    rows = np.sort(rng.choice(di, 48, replace=False))
+    cols = np.sort(rng.choice(n * dk, 48, replace=False))
+    A = a.reshape(dj, di)                         # A[j][i]
+    B = b.reshape(n * dk, dj)                     # B'[col][j]
+    GY = gy.reshape(n * dk, di)                   # gY'[col][i]
+    # y[rows, cols]
+    ref = oracle.matmul_fw(np.ascontiguousarray(A[:, rows]), np.ascontiguousarray(B[cols]),
+                           len(rows), dj, len(cols), 1, 1, 8).reshape(len(cols), len(rows))
+    assert norm_rel_err(y[np.ix_(cols, rows)], ref) <= w.tolerance
+    # ga[rows, jcols] = sum over all (col) gY'[rows, col] B'[jcols, col]
+    jc = np.sort(rng.choice(dj, 48, replace=False))
+    ref = (GY[:, rows].astype(np.float64).T @ B[:, jc].astype(np.float64)).T   # [j][i]
+    assert norm_rel_err(gav[np.ix_(jc, rows)], ref) <= w.tolerance
+    # gb[jcols, cols] = sum_i A[i, jcols] gY'[i, cols]
+    ref = (GY[cols].astype(np.float64) @ A[jc].astype(np.float64).T)           # [col][j]
+    assert norm_rel_err(gbv[np.ix_(cols, jc)], ref) <= w.tolerance
