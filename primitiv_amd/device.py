@@ -330,10 +330,10 @@ class HIP:
         return self._download(x.handle(), x.shape().size())
 
     def copy_tensor(self, x):
-        # devices/cuda/ops/copy_tensor.cu:10-30: same device type -> D2D,
+        # devices/cuda/ops/copy_tensor.cu:10-30: same storage type -> D2D,
         # anything else bounces through the host.
         ret = self.new_raw_tensor(x.shape())
-        if isinstance(x.device(), HIP) and x.device().type() == self.type():
+        if isinstance(x.device(), HIP) and x.device()._SUFFIX == self._SUFFIX:
             _lib.call("phip_memcpy_d2d", self._ctx, ret._handle.ptr, x.handle(),
                       self._elements_to_bytes(x.shape().size()))
         else:
