@@ -49,6 +49,14 @@ __device__ inline int xcd_remap(int bid, int total) {
   return xcd * q + (xcd < rem ? xcd : rem) + idx;
 }
 
+// The loaders below are branch-free so that the global loads of the next tile
+// can stay in flight while the matrix instructions of the current one run: a
+// vector that falls outside the matrix is read from the matrix origin instead
+// (always a valid address) and replaced by zeros when it is written to LDS.
+// With V == 4 the leading dimension is a multiple of 4, and so is the extent
+// along the contiguous axis (dense column-major: it IS the leading dimension),
+// so a vector is either entirely inside or entirely outside.
+
 // Tile of an operand that is contiguous along x (m or n): element (x, k) at
 // base[x + k*ld].  Rows of the LDS tile are k.
 template <int BX, int BK, int V>
@@ -57,22 +65,23 @@ struct LoaderXContig {
   static constexpr int kTotal = BX * BK / V;
   static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
   float regs[kIters][V];
+  unsigned ok;
 
   __device__ inline void load(const float *base, long ld, int x0, int X, int k0, int K, int tid) {
+    ok = 0;
 #pragma unroll
     for (int i = 0; i < kIters; ++i) {
       const int v = tid + i * kThreads;
       const int k = k0 + v / kVecPerRow;
       const int x = x0 + (v % kVecPerRow) * V;
-      const bool live = (kTotal % kThreads == 0 || v < kTotal) && k < K;
-      if (V == 4 && live && x + 4 <= X) {
-        const float4v t = *reinterpret_cast<const float4v *>(base + x + (long)k * ld);
+      const bool in = (kTotal % kThreads == 0 || v < kTotal) && k < K && x < X;
+      const float *p = in ? base + x + (long)k * ld : base;
+      ok |= (in ? 1u : 0u) << i;
+      if constexpr (V == 4) {
+        const float4v t = *reinterpret_cast<const float4v *>(p);
         regs[i][0] = t.x; regs[i][1 % V] = t.y; regs[i][2 % V] = t.z; regs[i][3 % V] = t.w;
       } else {
-#pragma unroll
-        for (int e = 0; e < V; ++e) {
-          regs[i][e] = (live && x + e < X) ? base[x + e + (long)k * ld] : 0.0f;
-        }
+        regs[i][0] = *p;
       }
     }
   }
@@ -83,13 +92,14 @@ struct LoaderXContig {
     for (int i = 0; i < kIters; ++i) {
       const int v = tid + i * kThreads;
       if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      const bool in = (ok >> i) & 1u;
       float *p = lds + (v / kVecPerRow) * S + (v % kVecPerRow) * V;
-      if (V == 4) {
-        float4v t = {regs[i][0], regs[i][1 % V], regs[i][2 % V], regs[i][3 % V]};
+      if constexpr (V == 4) {
+        float4v t = {in ? regs[i][0] : 0.0f, in ? regs[i][1 % V] : 0.0f, in ? regs[i][2 % V] : 0.0f,
+                     in ? regs[i][3 % V] : 0.0f};
         *reinterpret_cast<float4v *>(p) = t;
       } else {
-#pragma unroll
-        for (int e = 0; e < V; ++e) p[e] = regs[i][e];
+        p[0] = in ? regs[i][0] : 0.0f;
       }
     }
   }
@@ -103,22 +113,23 @@ struct LoaderKContig {
   static constexpr int kTotal = BX * BK / V;
   static constexpr int kIters = (kTotal + kThreads - 1) / kThreads;
   float regs[kIters][V];
+  unsigned ok;
 
   __device__ inline void load(const float *base, long ld, int x0, int X, int k0, int K, int tid) {
+    ok = 0;
 #pragma unroll
     for (int i = 0; i < kIters; ++i) {
       const int v = tid + i * kThreads;
       const int x = x0 + v / kVecPerX;
       const int k = k0 + (v % kVecPerX) * V;
-      const bool live = (kTotal % kThreads == 0 || v < kTotal) && x < X;
-      if (V == 4 && live && k + 4 <= K) {
-        const float4v t = *reinterpret_cast<const float4v *>(base + k + (long)x * ld);
+      const bool in = (kTotal % kThreads == 0 || v < kTotal) && x < X && k < K;
+      const float *p = in ? base + k + (long)x * ld : base;
+      ok |= (in ? 1u : 0u) << i;
+      if constexpr (V == 4) {
+        const float4v t = *reinterpret_cast<const float4v *>(p);
         regs[i][0] = t.x; regs[i][1 % V] = t.y; regs[i][2 % V] = t.z; regs[i][3 % V] = t.w;
       } else {
-#pragma unroll
-        for (int e = 0; e < V; ++e) {
-          regs[i][e] = (live && k + e < K) ? base[k + e + (long)x * ld] : 0.0f;
-        }
+        regs[i][0] = *p;
       }
     }
   }
@@ -129,9 +140,10 @@ struct LoaderKContig {
     for (int i = 0; i < kIters; ++i) {
       const int v = tid + i * kThreads;
       if (kTotal % kThreads != 0 && v >= kTotal) continue;
+      const bool in = (ok >> i) & 1u;
       float *p = lds + ((v % kVecPerX) * V) * S + v / kVecPerX;
 #pragma unroll
-      for (int e = 0; e < V; ++e) p[e * S] = regs[i][e];
+      for (int e = 0; e < V; ++e) p[e * S] = in ? regs[i][e] : 0.0f;
     }
   }
 };
@@ -148,8 +160,8 @@ struct LoaderSelect<true, BX, BK, V> {
 // WGM x WGN x WGK wavefronts: WGM*WGN of them tile the BM x BN block, WGK of
 // them share each wave tile and split the k steps of every K tile between
 // themselves (their partial tiles are summed through LDS at the end).
-template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool A_KMAJOR, bool B_KMAJOR, int V>
-__global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const GemmArgs g) {
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC, bool A_KMAJOR, bool B_KMAJOR, int V>
+__global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs g) {
   static_assert(WGM * WGN * WGK == 4, "four wavefronts per workgroup");
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -309,7 +321,7 @@ struct TileChoice {
   int bm, bn, bk;
 };
 
-template <int BM, int BN, int BK, int WGM, int WGN, int WGK>
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC>
 int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec4) {
   a.tiles_m = (p.M + BM - 1) / BM;
   a.tiles_n = (p.N + BN - 1) / BN;
@@ -342,7 +354,7 @@ int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec4) {
   }
 
 #define PHIP_LAUNCH(AK, BKM, VV)                                                                   \
-  hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VV>), dim3((unsigned)grid), \
+  hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WGM, WGN, WGK, OCC, AK, BKM, VV>), dim3((unsigned)grid), \
                      dim3(kThreads), 0, ctx->stream, a)
   if (!p.a_kmajor && p.b_kmajor) {
     if (vec4) PHIP_LAUNCH(false, true, 4); else PHIP_LAUNCH(false, true, 1);
@@ -376,15 +388,20 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   auto aligned = [](const void *ptr, long ld, long s, long r) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
   };
-  const bool vec4 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB);
+  // 16-byte loads need aligned rows and a contiguous-axis extent that is a
+  // multiple of 4 (so that no vector straddles the matrix edge).
+  const bool vec4 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB) &&
+                    (p.a_kmajor ? p.K : p.M) % 4 == 0 && (p.b_kmajor ? p.K : p.N) % 4 == 0;
 
   const int cus = ctx->prop.multiProcessorCount;
   auto tiles = [&](int bm, int bn) {
     return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch;
   };
-  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1>(ctx, p, a, vec4);
-  if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1>(ctx, p, a, vec4);
-  return launch_tile<32, 32, 64, 1, 1, 4>(ctx, p, a, vec4);
+  // 128x128x16 at four workgroups per CU (33 KiB of LDS and 128 VGPRs each)
+  // measured fastest among BK 8/16/32 and 2..4 workgroups per CU.
+  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, a, vec4);
+  if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, a, vec4);
+  return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, a, vec4);
 }
 
 }  // namespace phip
