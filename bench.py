@@ -30,6 +30,10 @@ from primitiv_amd.configs import WORKLOADS  # noqa: E402
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6, "bf16": 2516.6}
 PEAK_HBM_GBS = 8000.0
 HEADLINE = "square_batched"
+# HBM bytes per launch of the headline kernel (average of its three operand-layout
+# instantiations): rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors read
+# off a streaming y += x of known size (the summary under profiles/ holds both runs).
+HEADLINE_TRAFFIC_BYTES = 220.2e6 + 73.4e6
 
 
 class Resident:
@@ -150,10 +154,22 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all", help="all or one of: " + ", ".join(WORKLOADS))
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="first run one streaming y += x over 64 Mi floats (reads 512 MiB, writes 256 MiB): "
+                         "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path "
                  "(run with --gpus 1).")
+
+    if args.traffic_calibration:
+        dev = pa.HIP(0)
+        n = 64 << 20
+        x, y = dev.new_tensor_by_constant([n], 1.0), dev.new_tensor_by_constant([n], 2.0)
+        y += x
+        dev.sync()
+        del x, y
+        dev.close()
 
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     if HEADLINE not in names and args.workload == "all":
@@ -176,7 +192,7 @@ def main():
     roofline = {
         "bound": "mfma", "achieved": flops_per_launch / launch_s / 1e12, "peak": PEAK_TFLOPS[w.storage],
         "unit": "TFLOP/s", "frac": flops_per_launch / launch_s / 1e12 / PEAK_TFLOPS[w.storage],
-        "traffic": None,
+        "traffic": HEADLINE_TRAFFIC_BYTES if head["workload"] == HEADLINE else None,
         "kernel": "gemm_f32_kernel<128,128,16,...> (fw NN, gA NT, gB TN)",
         "flops_per_launch": flops_per_launch, "avg_launch_ms": launch_s * 1e3,
     }

@@ -1,0 +1,70 @@
+# Build fragment for primitiv's PRIMITIV_USE_HIP option (AMD MI355X, gfx950).
+#
+# How it plugs into primitiv's own build (primitiv v0.4.0):
+#   * top-level CMakeLists.txt, next to the other backend options (lines 13-16):
+#       option(PRIMITIV_USE_HIP "Enable the MI355X (gfx950) HIP backend." OFF)
+#   * primitiv/config.h.in, next to PRIMITIV_USE_CUDA:
+#       #cmakedefine PRIMITIV_USE_HIP
+#   * primitiv/CMakeLists.txt, after the CUDA block (lines 125-187):
+#       if(PRIMITIV_USE_HIP)
+#         include(${PRIMITIV_HIP_BACKEND_DIR}/primitiv/cmake/hip_backend.cmake)
+#       endif()
+#     where PRIMITIV_HIP_BACKEND_DIR points at the directory that holds this
+#     backend's `primitiv/` and `csrc/` folders and `include/phip.h`.
+#
+# The fragment builds libphip (HIP device code, gfx950 only) with hipcc and
+# adds the host-side devices::HIP class and its C-API constructor to the
+# object lists that primitiv folds into libprimitiv.
+
+if(NOT DEFINED PRIMITIV_HIP_BACKEND_DIR)
+  get_filename_component(PRIMITIV_HIP_BACKEND_DIR "${CMAKE_CURRENT_LIST_DIR}/../.." ABSOLUTE)
+endif()
+if(NOT DEFINED PRIMITIV_HIP_PHIP_INCLUDE_DIR)
+  get_filename_component(PRIMITIV_HIP_PHIP_INCLUDE_DIR "${PRIMITIV_HIP_BACKEND_DIR}/../include" ABSOLUTE)
+endif()
+if(NOT DEFINED ROCM_PATH)
+  set(ROCM_PATH "/opt/rocm")
+endif()
+find_program(PRIMITIV_HIPCC hipcc HINTS "${ROCM_PATH}/bin" REQUIRED)
+
+set(phip_SRCS
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_runtime.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_elementwise.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_matmul.hip
+)
+set(phip_LIB ${CMAKE_CURRENT_BINARY_DIR}/libphip.so)
+add_custom_command(
+  OUTPUT ${phip_LIB}
+  COMMAND ${PRIMITIV_HIPCC} --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared
+          -Xclang -target-feature -Xclang -packed-fp32-ops
+          -I${PRIMITIV_HIP_PHIP_INCLUDE_DIR} ${phip_SRCS} -o ${phip_LIB}
+  DEPENDS ${phip_SRCS}
+  COMMENT "Building libphip (HIP kernels for gfx950)"
+)
+add_custom_target(phip ALL DEPENDS ${phip_LIB})
+install(FILES ${phip_LIB} DESTINATION ${CMAKE_INSTALL_LIBDIR})
+install(FILES ${PRIMITIV_HIP_PHIP_INCLUDE_DIR}/phip.h DESTINATION ${CMAKE_INSTALL_INCLUDEDIR})
+
+# Host-side device class (plain C++11, compiled by the project's compiler).
+file(GLOB primitiv_hip_HDRS "${PRIMITIV_HIP_BACKEND_DIR}/primitiv/devices/hip/*.h")
+file(GLOB primitiv_hip_SRCS "${PRIMITIV_HIP_BACKEND_DIR}/primitiv/devices/hip/*.cc")
+add_library(primitiv_hip_OBJS OBJECT ${primitiv_hip_HDRS} ${primitiv_hip_SRCS})
+target_include_directories(primitiv_hip_OBJS PRIVATE
+  ${PRIMITIV_HIP_BACKEND_DIR} ${PRIMITIV_HIP_PHIP_INCLUDE_DIR})
+add_dependencies(primitiv_hip_OBJS phip)
+list(APPEND primitiv_all_OBJS $<TARGET_OBJECTS:primitiv_hip_OBJS>)
+list(APPEND primitiv_all_DEPS ${phip_LIB})
+install(FILES ${primitiv_hip_HDRS} DESTINATION ${CMAKE_INSTALL_INCLUDEDIR}/primitiv/devices/hip)
+
+# C API constructor (same switch as the other backends, primitiv/CMakeLists.txt:285-297).
+if(PRIMITIV_BUILD_C_API)
+  file(GLOB primitiv_c_hip_HDRS "${PRIMITIV_HIP_BACKEND_DIR}/primitiv/c/devices/hip/*.h")
+  file(GLOB primitiv_c_hip_SRCS "${PRIMITIV_HIP_BACKEND_DIR}/primitiv/c/devices/hip/*.cc")
+  add_library(primitiv_c_hip_OBJS OBJECT ${primitiv_c_hip_HDRS} ${primitiv_c_hip_SRCS})
+  target_include_directories(primitiv_c_hip_OBJS PRIVATE
+    ${PRIMITIV_HIP_BACKEND_DIR} ${PRIMITIV_HIP_PHIP_INCLUDE_DIR})
+  list(APPEND primitiv_all_OBJS $<TARGET_OBJECTS:primitiv_c_hip_OBJS>)
+  install(FILES ${primitiv_c_hip_HDRS} DESTINATION ${CMAKE_INSTALL_INCLUDEDIR}/primitiv/c/devices/hip)
+endif()

@@ -1,0 +1,192 @@
+#ifndef PRIMITIV_DEVICES_HIP_DEVICE_H_
+#define PRIMITIV_DEVICES_HIP_DEVICE_H_
+
+// primitiv::devices::HIP -- AMD MI355X (gfx950) backend for the matmul path.
+//
+// Drop-in subclass of primitiv::Device (primitiv/core/device.h): the existing
+// Graph / Node / Tensor / Parameter code talks to it through the same virtual
+// interface as to the CUDA backend (primitiv/devices/cuda/device.h).  All GPU
+// work goes through libphip's C ABI (phip.h); this class only owns the
+// context and the memory pool and forwards each operation.
+//
+// Implemented: matmul forward/backward and the helpers the graph needs around
+// them (allocation, fill, host<->device and device<->device copies, in-place
+// add with minibatch broadcasting, minibatch sum).  Every other operation
+// throws primitiv::NotImplementedError, as the reference's own backends do for
+// operations they lack (primitiv/devices/opencl/ops/conv2d.cc:16,25).
+
+#include <cstdint>
+#include <memory>
+#include <vector>
+
+#include <primitiv/core/device.h>
+#include <primitiv/core/error.h>
+#include <primitiv/core/memory_pool.h>
+
+struct phip_ctx;
+
+namespace primitiv {
+namespace devices {
+
+// Values to be added to enum DeviceType (primitiv/core/device.h:17-35) as a
+// fourth group; spelled as casts here so that this header also compiles
+// against an unpatched primitiv.
+constexpr DeviceType DEVICE_TYPE_GROUP_HIP = static_cast<DeviceType>(0x00030000u);
+constexpr DeviceType DEVICE_TYPE_HIP = static_cast<DeviceType>(0x00030000u);
+constexpr DeviceType DEVICE_TYPE_HIP16 = static_cast<DeviceType>(0x00030001u);
+
+class HIP : public Device {
+public:
+  // Element type of tensors in device memory.  The public API is float in
+  // every case; F16 / BF16 store 16-bit values and accumulate in fp32 (the
+  // counterpart of devices::CUDA16, primitiv/devices/cuda16/device.h).
+  enum class Storage : std::uint32_t { F32 = 0, F16 = 1, BF16 = 2 };
+
+  // Number of HIP devices visible to this process.
+  static std::uint32_t num_devices();
+
+  // Throws primitiv::Error unless `device_id` exists and is a gfx950 device
+  // with 64-wide wavefronts and at least 1 GiB of memory.
+  static void assert_support(std::uint32_t device_id);
+
+  // Same test as assert_support, reported as a boolean.
+  static bool check_support(std::uint32_t device_id);
+
+  explicit HIP(std::uint32_t device_id);
+  HIP(std::uint32_t device_id, std::uint32_t rng_seed);
+  HIP(std::uint32_t device_id, std::uint32_t rng_seed, Storage storage);
+  ~HIP() override;
+
+  void dump_description() const override;
+  DeviceType type() const override {
+    return storage_ == Storage::F32 ? DEVICE_TYPE_HIP : DEVICE_TYPE_HIP16;
+  }
+  Storage storage() const { return storage_; }
+
+private:
+  // ---- implemented -------------------------------------------------------
+  std::shared_ptr<void> new_handle(const Shape &shape, std::size_t *const allocated_size) override;
+  std::vector<float> tensor_to_vector_impl(const Tensor &x) override;
+  void reset_tensor_impl(float k, Tensor &x) override;
+  void reset_tensor_by_array_impl(const float values[], Tensor &x) override;
+  void copy_tensor_impl(const Tensor &x, Tensor &y) override;
+  void identity_impl(Tensor &y) override;
+  void matmul_fw_impl(const Tensor &a, const Tensor &b, Tensor &y) override;
+  void matmul_bw_impl(const Tensor &a, const Tensor &b, const Tensor &y, const Tensor &gy,
+                      Tensor &ga, Tensor &gb) override;
+  void batch_sum_fw_impl(const Tensor &x, Tensor &y) override;
+  void inplace_add_impl(const Tensor &x, Tensor &y) override;
+
+  // ---- not implemented in this backend -------------------------------------
+  [[noreturn]] static void unsupported(const char *op);
+
+#define PHIP_NI_X(name) \
+  void name##_impl(const Tensor &, Tensor &) override { unsupported(#name); }
+#define PHIP_NI_X_BW(name) \
+  void name##_impl(const Tensor &, const Tensor &, const Tensor &, Tensor &) override { unsupported(#name); }
+#define PHIP_NI_CONST(name, K) \
+  void name##_fw_impl(const Tensor &, K, Tensor &) override { unsupported(#name "_fw"); } \
+  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, K, Tensor &) override { unsupported(#name "_bw"); }
+#define PHIP_NI_SCALAR(name) \
+  void name##_fw_impl(const Tensor &, const Tensor &, Tensor &) override { unsupported(#name "_fw"); }
+#define PHIP_NI_AB(name) \
+  void name##_fw_impl(const Tensor &, const Tensor &, Tensor &) override { unsupported(#name "_fw"); } \
+  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, const Tensor &, Tensor &, Tensor &) override { unsupported(#name "_bw"); }
+#define PHIP_NI_DIM(name) \
+  void name##_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported(#name "_fw"); }
+#define PHIP_NI_DIM_BW(name) \
+  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, std::uint32_t, Tensor &) override { unsupported(#name "_bw"); }
+#define PHIP_NI_RANDOM(name) \
+  void random_##name##_impl(float, float, Tensor &) override { unsupported("random_" #name); }
+
+  std::vector<std::uint32_t> argmax_impl(const Tensor &, std::uint32_t) override { unsupported("argmax"); }
+  std::vector<std::uint32_t> argmin_impl(const Tensor &, std::uint32_t) override { unsupported("argmin"); }
+  void random_bernoulli_impl(float, Tensor &) override { unsupported("random_bernoulli"); }
+  PHIP_NI_RANDOM(uniform) PHIP_NI_RANDOM(normal) PHIP_NI_RANDOM(log_normal)
+
+  void pick_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, std::uint32_t, Tensor &) override { unsupported("pick_fw"); }
+  void slice_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("slice_fw"); }
+  void concat_fw_impl(const std::vector<const Tensor *> &, std::uint32_t, Tensor &) override { unsupported("concat_fw"); }
+  void pick_bw_impl(const Tensor &, const std::vector<std::uint32_t> &, std::uint32_t, Tensor &) override { unsupported("pick_bw"); }
+  void slice_bw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("slice_bw"); }
+
+  PHIP_NI_X(negate_fw) PHIP_NI_X(abs_fw) PHIP_NI_X(sqrt_fw) PHIP_NI_X(exp_fw) PHIP_NI_X(log_fw)
+  PHIP_NI_X(tanh_fw) PHIP_NI_X(sigmoid_fw) PHIP_NI_X(softplus_fw) PHIP_NI_X(sin_fw) PHIP_NI_X(cos_fw)
+  PHIP_NI_X(tan_fw) PHIP_NI_X(transpose_fw)
+  void permute_dims_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_fw"); }
+  void flip_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_fw"); }
+
+  PHIP_NI_X_BW(abs_bw) PHIP_NI_X_BW(sqrt_bw) PHIP_NI_X_BW(exp_bw) PHIP_NI_X_BW(log_bw) PHIP_NI_X_BW(tanh_bw)
+  PHIP_NI_X_BW(sigmoid_bw) PHIP_NI_X_BW(softplus_bw) PHIP_NI_X_BW(sin_bw) PHIP_NI_X_BW(cos_bw)
+  PHIP_NI_X_BW(tan_bw) PHIP_NI_X_BW(transpose_bw)
+  void permute_dims_bw_impl(const Tensor &, const Tensor &, const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_bw"); }
+  void flip_bw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_bw"); }
+
+  PHIP_NI_CONST(add_const, float) PHIP_NI_CONST(subtract_const_r, float) PHIP_NI_CONST(subtract_const_l, float)
+  PHIP_NI_CONST(multiply_const, float) PHIP_NI_CONST(divide_const_r, float) PHIP_NI_CONST(divide_const_l, float)
+  PHIP_NI_CONST(pow_const_r, float) PHIP_NI_CONST(pow_const_l, float) PHIP_NI_CONST(prelu, float)
+  PHIP_NI_CONST(elu, float) PHIP_NI_CONST(pown, std::int32_t)
+
+  PHIP_NI_SCALAR(add_scalar) PHIP_NI_SCALAR(subtract_scalar_r) PHIP_NI_SCALAR(subtract_scalar_l)
+  PHIP_NI_SCALAR(multiply_scalar) PHIP_NI_SCALAR(divide_scalar_r) PHIP_NI_SCALAR(divide_scalar_l)
+  PHIP_NI_SCALAR(pow_scalar_r) PHIP_NI_SCALAR(pow_scalar_l)
+
+  PHIP_NI_AB(add) PHIP_NI_AB(subtract) PHIP_NI_AB(multiply) PHIP_NI_AB(divide) PHIP_NI_AB(pow)
+
+  PHIP_NI_DIM(max) PHIP_NI_DIM(min) PHIP_NI_DIM(sum) PHIP_NI_DIM(logsumexp)
+  PHIP_NI_DIM_BW(max) PHIP_NI_DIM_BW(min)
+  void broadcast_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("broadcast_fw"); }
+
+  void batch_pick_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("batch_pick_fw"); }
+  void batch_slice_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("batch_slice_fw"); }
+  void batch_concat_fw_impl(const std::vector<const Tensor *> &, Tensor &) override { unsupported("batch_concat_fw"); }
+  void batch_pick_bw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("batch_pick_bw"); }
+  void batch_slice_bw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("batch_slice_bw"); }
+
+  void conv2d_fw_impl(const Tensor &, const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t,
+                      std::uint32_t, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("conv2d_fw"); }
+  void conv2d_bw_impl(const Tensor &, const Tensor &, const Tensor &, const Tensor &, std::uint32_t,
+                      std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
+                      Tensor &, Tensor &) override { unsupported("conv2d_bw"); }
+  void max_pool2d_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
+                          std::uint32_t, std::uint32_t, Tensor &) override { unsupported("max_pool2d_fw"); }
+  void max_pool2d_bw_impl(const Tensor &, const Tensor &, const Tensor &, std::uint32_t, std::uint32_t,
+                          std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
+                          Tensor &) override { unsupported("max_pool2d_bw"); }
+
+  void inplace_multiply_const_impl(float, Tensor &) override { unsupported("inplace_multiply_const"); }
+  void inplace_subtract_impl(const Tensor &, Tensor &) override { unsupported("inplace_subtract"); }
+
+#undef PHIP_NI_X
+#undef PHIP_NI_X_BW
+#undef PHIP_NI_CONST
+#undef PHIP_NI_SCALAR
+#undef PHIP_NI_AB
+#undef PHIP_NI_DIM
+#undef PHIP_NI_DIM_BW
+#undef PHIP_NI_RANDOM
+
+  // Bytes of device storage for `n` elements (16-bit storage rounds the
+  // element count up to even, as devices::CUDA16 does).
+  std::size_t storage_bytes(std::size_t n) const;
+
+  std::uint32_t dev_id_;
+  std::uint32_t rng_seed_;
+  Storage storage_;
+  // Declared before the pool so that it is destroyed after it: the pool's
+  // deleter still needs the context while it frees its blocks.
+  phip_ctx *ctx_;
+  std::unique_ptr<MemoryPool> pool_;
+};
+
+// Half-storage device with the constructor shape of devices::CUDA16.
+class HIP16 : public HIP {
+public:
+  explicit HIP16(std::uint32_t device_id);
+  HIP16(std::uint32_t device_id, std::uint32_t rng_seed);
+};
+
+}  // namespace devices
+}  // namespace primitiv
+
+#endif  // PRIMITIV_DEVICES_HIP_DEVICE_H_
