@@ -183,6 +183,46 @@ def test_random_shapes_h16(dev16, devbf16, which, ba, bb):
                 assert norm_rel_err(got, ref) <= tol, name + " " + tag
 
 
+# shapes that reach the 256x256x64 large-tile kernel with ragged edges in every
+# dimension (multiples of 8, not of 256 / 64), in each batch case
+BIG_H16 = [  # di, dj, dk, ba, bb
+    (2824, 2832, 2840, 1, 1),
+    (776, 520, 1032, 16, 16),
+    (136, 2824, 2832, 16, 1),
+    (2824, 264, 712, 1, 4),
+]
+
+
+@pytest.mark.parametrize("which", ["f16", "bf16"])
+@pytest.mark.parametrize("di,dj,dk,ba,bb", BIG_H16)
+def test_large_tile_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
+    d = dev16 if which == "f16" else devbf16
+    rng = np.random.default_rng(di + dj + dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(y, ry) <= H16_TOL
+    assert norm_rel_err(ga, rga) <= H16_TOL
+    assert norm_rel_err(gb, rgb) <= H16_TOL
+    # inputs exactly representable in 16 bits: only the output rounding is left
+    r16 = (lambda x: x.astype(np.float16).astype(np.float32)) if which == "f16" else \
+        (lambda x: (x.view(np.uint32) & 0xFFFF0000).view(np.float32))
+    a, b, gy = r16(a), r16(b), r16(gy)
+    z = lambda n: np.zeros(n, dtype=np.float32)
+    y, ga, gb = _fw_bw(d, a, b, gy, z(a.size), z(b.size), di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, z(a.size), z(b.size), di, dj, dk, ba, bb, 8)
+    ulp = 2.0 ** -10 if which == "f16" else 2.0 ** -7
+    for got, ref in ((y, ry), (ga, rga), (gb, rgb)):
+        assert norm_rel_err(got, ref) <= ulp
+
+
 def test_f16_matches_oracle_on_rounded_inputs(dev16):
     # With inputs already representable in fp16 the only error left is the
     # final rounding of the output (<= 2^-11 relative per element) on top of
