@@ -90,37 +90,45 @@ struct TileLoader {
     }
   }
 
+  // Prepares tile `kt_in_r` of the current sample; `live` false turns every
+  // load of the tile into an out-of-range one (reads zeros, touches nothing).
+  uint32_t adv;
+  bool in;
+  __device__ inline void begin(int kt_in_r, int K, bool live) {
+    adv = (uint32_t)kt_in_r * step;
+    if constexpr (KMAJOR) in = live && kt_in_r * BK + kg * 8 < K;  // the next column starts right after K
+    else in = live && x_in;                                         // rows past K are past the end
+  }
+  __device__ inline void load_one(__amdgpu_buffer_rsrc_t rsrc, int i) {
+    const uint32_t o = in ? off[i] + adv : kOutOfRange;
+    regs[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)o, 0, 0);
+  }
   __device__ inline void load(__amdgpu_buffer_rsrc_t rsrc, int kt_in_r, int K) {
-    const uint32_t adv = (uint32_t)kt_in_r * step;
-    bool in;
-    if constexpr (KMAJOR) in = kt_in_r * BK + kg * 8 < K;  // the next column starts right after K
-    else in = x_in;                                         // rows past K are past the end
+    begin(kt_in_r, K, true);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t o = in ? off[i] + adv : kOutOfRange;
-      regs[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)o, 0, 0);
-    }
+    for (int i = 0; i < 8; ++i) load_one(rsrc, i);
   }
 
-  __device__ inline void store(uint16_t *lds) const {
+  // Writes the j-th of this thread's eight 16-byte LDS row segments.
+  __device__ inline void store_one(uint16_t *lds, int j) const {
     uint16_t *p = lds + lds_off;
     if constexpr (KMAJOR) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4v *>(p + 32 * i * S) = regs[i];
+      *reinterpret_cast<uint4v *>(p + 32 * j * S) = regs[j];
     } else {
       // regs[i] = 8 columns of k row i.  Output row j = column j across the 8
       // k rows: dword d of it packs (row 2d, row 2d+1) of element j.
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-        uint4v o;
-        o.x = __builtin_amdgcn_perm(regs[1][j >> 1], regs[0][j >> 1], sel);
-        o.y = __builtin_amdgcn_perm(regs[3][j >> 1], regs[2][j >> 1], sel);
-        o.z = __builtin_amdgcn_perm(regs[5][j >> 1], regs[4][j >> 1], sel);
-        o.w = __builtin_amdgcn_perm(regs[7][j >> 1], regs[6][j >> 1], sel);
-        *reinterpret_cast<uint4v *>(p + j * S) = o;
-      }
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      uint4v o;
+      o.x = __builtin_amdgcn_perm(regs[1][j >> 1], regs[0][j >> 1], sel);
+      o.y = __builtin_amdgcn_perm(regs[3][j >> 1], regs[2][j >> 1], sel);
+      o.z = __builtin_amdgcn_perm(regs[5][j >> 1], regs[4][j >> 1], sel);
+      o.w = __builtin_amdgcn_perm(regs[7][j >> 1], regs[6][j >> 1], sel);
+      *reinterpret_cast<uint4v *>(p + j * S) = o;
     }
+  }
+  __device__ inline void store(uint16_t *lds) const {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) store_one(lds, j);
   }
 };
 
@@ -189,48 +197,67 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_big_kernel(const BigArgs
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  auto fetch = [&](int kt) {
-    const int r = kt / g.ktiles_per_r;
-    const int kt_in_r = kt - r * g.ktiles_per_r;
-    la.load(make_rsrc(Az + (long)r * g.rA, g.a_bytes), kt_in_r, g.K);
-    lb.load(make_rsrc(Bz + (long)r * g.rB, g.b_bytes), kt_in_r, g.K);
-  };
-
   const int kt_end = g.total_ktiles;
-  if (kt_end > 0) {
-    fetch(0);
+  {
+    la.load(make_rsrc(Az, g.a_bytes), 0, g.K);
+    lb.load(make_rsrc(Bz, g.b_bytes), 0, g.K);
     la.store(lds);
     lb.store(lds + 2 * kStageA);
   }
   __syncthreads();
 
-  // lane l supplies row l%32 and the 8 k values starting at 8*(l/32)
+  // Lane l supplies row l%32 and the 8 k values starting at 8*(l/32).
   const int frag_off = (lane & 31) * S + 8 * (lane >> 5);
+  const uint16_t *a_frag = lds + wm * 128 * S + frag_off;
+  const uint16_t *b_frag = lds + 2 * kStageA + wn * 128 * S + frag_off;
+
+  // Fragments are double-buffered in registers: the reads of k step s+1 are
+  // issued between the matrix instructions of step s, and the first step of
+  // the next tile is read behind the barrier, under the last step of this one.
+  uint4v fa[2][4], fb[2][4];
+  auto read_frag = [&](int buf, int q, int stage, int s) {
+    if (q < 4) fa[buf][q] = *reinterpret_cast<const uint4v *>(a_frag + stage * kStageA + q * 32 * S + s * 16);
+    else fb[buf][q - 4] = *reinterpret_cast<const uint4v *>(b_frag + stage * kStageB + (q - 4) * 32 * S + s * 16);
+  };
+#pragma unroll
+  for (int q = 0; q < 8; ++q) read_frag(0, q, 0, 0);
+
   for (int kt = 0; kt < kt_end; ++kt) {
     const int stage = kt & 1;
+    // Next tile (loads degenerate to out-of-range reads after the last one).
     const bool more = kt + 1 < kt_end;
-    if (more) fetch(kt + 1);
+    const int nkt = more ? kt + 1 : kt;
+    const int r = nkt / g.ktiles_per_r;
+    const int kt_in_r = nkt - r * g.ktiles_per_r;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Az + (long)r * g.rA, g.a_bytes);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bz + (long)r * g.rB, g.b_bytes);
+    la.begin(kt_in_r, g.K, more);
+    lb.begin(kt_in_r, g.K, more);
+    uint16_t *next_a = lds + (stage ^ 1) * kStageA;
+    uint16_t *next_b = lds + 2 * kStageA + (stage ^ 1) * kStageB;
 
-    const uint16_t *as = lds + stage * kStageA + wm * 128 * S + frag_off;
-    const uint16_t *bs = lds + 2 * kStageA + stage * kStageB + wn * 128 * S + frag_off;
 #pragma unroll
-    for (int s = 0; s < BK / 16; ++s) {
-      uint4v af[4], bf[4];
+    for (int s = 0; s < 4; ++s) {
+      const int cur = s & 1, nxt = cur ^ 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const uint4v *>(as + i * 32 * S + s * 16);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const uint4v *>(bs + j * 32 * S + s * 16);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma<BF16>(bf[j], af[i], acc[i][j]);
+      for (int q = 0; q < 16; ++q) {
+        const int i = q >> 2, j = q & 3;
+        acc[i][j] = mfma<BF16>(fb[cur][j], fa[cur][i], acc[i][j]);
+        // work slotted in behind this matrix instruction
+        if (s == 0) {
+          if (q < 8) la.load_one(ra, q); else lb.load_one(rb, q - 8);
+        }
+        if (q < 8) {
+          if (s < 3) read_frag(nxt, q, stage, s + 1);
+          else read_frag(nxt, q, stage ^ 1, 0);
+        }
+        if (s == 2) {
+          if (q < 8) la.store_one(next_a, q); else lb.store_one(next_b, q - 8);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (s == 2) __syncthreads();
     }
-
-    if (more) {
-      la.store(lds + (stage ^ 1) * kStageA);
-      lb.store(lds + 2 * kStageA + (stage ^ 1) * kStageB);
-    }
-    __syncthreads();
   }
 
   // Lane l of result register v holds C(m, n) with m = l % 32 and
