@@ -157,10 +157,70 @@ struct LoaderSelect<true, BX, BK, V> {
   typedef LoaderKContig<BX, BK, V> type;
 };
 
+// Writes NV results of one lane into C.  Result q belongs to row m and column
+// ncol + nq[q], where (m, ncol) = (row0 + lane%32, col0 + 4*(lane/32)) and nq[]
+// is the same for all lanes.  The old values of an accumulating write are
+// fetched first, all NV loads in flight together.
+//  * Interior tiles: every address is a wave-uniform base (row0, col0 + nq[q])
+//    plus one per-lane 32-bit offset, no predicates.
+//  * Edge tiles: per-element predicates; an element outside the matrix reads
+//    the matrix origin instead and is not stored.
+template <int NV>
+__device__ inline void emit_c(float *Cz, long ldc, int row0, int col0, int lane, int M, int N, bool interior,
+                              const int (&nq)[NV], const float (&vals)[NV], int atomic, int accumulate) {
+  if (interior) {
+    const unsigned voff = (unsigned)((lane & 31) + 4L * (lane >> 5) * ldc);
+    float *base[NV];
+#pragma unroll
+    for (int q = 0; q < NV; ++q) base[q] = Cz + row0 + (long)(col0 + nq[q]) * ldc;  // uniform
+    if (atomic) {
+#pragma unroll
+      for (int q = 0; q < NV; ++q) unsafeAtomicAdd(base[q] + voff, vals[q]);
+    } else if (accumulate) {
+      float old[NV];
+#pragma unroll
+      for (int q = 0; q < NV; ++q) old[q] = base[q][voff];
+#pragma unroll
+      for (int q = 0; q < NV; ++q) base[q][voff] = old[q] + vals[q];
+    } else {
+#pragma unroll
+      for (int q = 0; q < NV; ++q) base[q][voff] = vals[q];
+    }
+    return;
+  }
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+  constexpr int kChunk = NV < 4 ? NV : 4;  // few live addresses: this path is rare
+#pragma unroll
+  for (int c = 0; c < NV; c += kChunk) {
+    bool ok[kChunk];
+    float *p[kChunk];
+    float old[kChunk];
+#pragma unroll
+    for (int q = 0; q < kChunk; ++q) {
+      ok[q] = m < M && ncol + nq[c + q] < N;
+      p[q] = ok[q] ? Cz + m + (long)(ncol + nq[c + q]) * ldc : Cz;
+    }
+    if (atomic) {
+#pragma unroll
+      for (int q = 0; q < kChunk; ++q)
+        if (ok[q]) unsafeAtomicAdd(p[q], vals[c + q]);
+    } else {
+      if (accumulate) {
+#pragma unroll
+        for (int q = 0; q < kChunk; ++q) old[q] = *p[q];
+      }
+#pragma unroll
+      for (int q = 0; q < kChunk; ++q)
+        if (ok[q]) *p[q] = accumulate ? old[q] + vals[c + q] : vals[c + q];
+    }
+  }
+}
+
 // WGM x WGN x WGK wavefronts: WGM*WGN of them tile the BM x BN block, WGK of
 // them share each wave tile and split the k steps of every K tile between
 // themselves (their partial tiles are summed through LDS at the end).
-template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC, bool A_KMAJOR, bool B_KMAJOR, int V>
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC, bool A_KMAJOR, bool B_KMAJOR, int VA, int VB>
 __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs g) {
   static_assert(WGM * WGN * WGK == 4, "four wavefronts per workgroup");
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -194,8 +254,8 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs 
   const float *Az = g.A + (long)z * g.sA;
   const float *Bz = g.B + (long)z * g.sB;
 
-  typename LoaderSelect<A_KMAJOR, BM, BK, V>::type la;
-  typename LoaderSelect<B_KMAJOR, BN, BK, V>::type lb;
+  typename LoaderSelect<A_KMAJOR, BM, BK, VA>::type la;
+  typename LoaderSelect<B_KMAJOR, BN, BK, VB>::type lb;
 
   float16v acc[TM][TN];
 #pragma unroll
@@ -253,8 +313,8 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs 
   // Lane l of result register v holds C(m, n) with m = l % 32 and
   // n = 8*(v/4) + 4*(l/32) + v%4 inside its 32x32 block.
   float *Cz = g.C + (long)z * g.sC;
-  const int cm = m0 + wm * WTM + (lane & 31);
-  const int cn = n0 + wn * WTN + 4 * (lane >> 5);
+  const int row0 = m0 + wm * WTM, col0 = n0 + wn * WTN;
+  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
 
   if (WGK > 1) {
     // Sum the k-split waves' tiles: every wave parks its registers in LDS,
@@ -273,7 +333,9 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs 
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j) {
+        float vals[kPer];
+        int ns[kPer];
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
           const int v = wk * kPer + q;
@@ -281,30 +343,27 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs 
 #pragma unroll
           for (int w = 0; w < WGK; ++w)
             s += red[((((group * WGK + w) * TM + i) * TN + j) * 16 + v) * 64 + lane];
-          const int m = cm + i * 32;
-          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
-          if (m < g.M && n < g.N) {
-            float *p = Cz + m + (long)n * g.ldc;
-            if (g.atomic) unsafeAtomicAdd(p, s);
-            else *p = g.accumulate ? *p + s : s;
-          }
+          vals[q] = s;
+          ns[q] = 8 * (v / 4) + (v % 4);
         }
+        emit_c<kPer>(Cz, g.ldc, row0 + i * 32, col0 + j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic,
+                     g.accumulate);
+      }
   } else {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j) {
+        float vals[16];
+        int ns[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int m = cm + i * 32;
-          const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
-          if (m < g.M && n < g.N) {
-            float *p = Cz + m + (long)n * g.ldc;
-            const float s = acc[i][j][v];
-            if (g.atomic) unsafeAtomicAdd(p, s);
-            else *p = g.accumulate ? *p + s : s;
-          }
+          vals[v] = acc[i][j][v];
+          ns[v] = 8 * (v / 4) + (v % 4);
         }
+        emit_c<16>(Cz, g.ldc, row0 + i * 32, col0 + j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic,
+                   g.accumulate);
+      }
   }
 }
 
@@ -322,7 +381,7 @@ struct TileChoice {
 };
 
 template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC>
-int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec4) {
+int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec_a, bool vec_b) {
   a.tiles_m = (p.M + BM - 1) / BM;
   a.tiles_n = (p.N + BN - 1) / BN;
   a.ktiles_per_r = (p.K + BK - 1) / BK;
@@ -353,18 +412,26 @@ int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec4) {
     PHIP_LAUNCH_CHECK();
   }
 
-#define PHIP_LAUNCH(AK, BKM, VV)                                                                   \
-  hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WGM, WGN, WGK, OCC, AK, BKM, VV>), dim3((unsigned)grid), \
-                     dim3(kThreads), 0, ctx->stream, a)
+#define PHIP_LAUNCH_V(AK, BKM, VVA, VVB)                                                            \
+  hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WGM, WGN, WGK, OCC, AK, BKM, VVA, VVB>),            \
+                     dim3((unsigned)grid), dim3(kThreads), 0, ctx->stream, a)
+#define PHIP_LAUNCH(AK, BKM)                                                                        \
+  do {                                                                                              \
+    if (vec_a && vec_b) PHIP_LAUNCH_V(AK, BKM, 4, 4);                                               \
+    else if (vec_a) PHIP_LAUNCH_V(AK, BKM, 4, 1);                                                   \
+    else if (vec_b) PHIP_LAUNCH_V(AK, BKM, 1, 4);                                                   \
+    else PHIP_LAUNCH_V(AK, BKM, 1, 1);                                                              \
+  } while (0)
   if (!p.a_kmajor && p.b_kmajor) {
-    if (vec4) PHIP_LAUNCH(false, true, 4); else PHIP_LAUNCH(false, true, 1);
+    PHIP_LAUNCH(false, true);
   } else if (!p.a_kmajor && !p.b_kmajor) {
-    if (vec4) PHIP_LAUNCH(false, false, 4); else PHIP_LAUNCH(false, false, 1);
+    PHIP_LAUNCH(false, false);
   } else if (p.a_kmajor && p.b_kmajor) {
-    if (vec4) PHIP_LAUNCH(true, true, 4); else PHIP_LAUNCH(true, true, 1);
+    PHIP_LAUNCH(true, true);
   } else {
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
+#undef PHIP_LAUNCH_V
 #undef PHIP_LAUNCH
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
@@ -390,8 +457,8 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   };
   // 16-byte loads need aligned rows and a contiguous-axis extent that is a
   // multiple of 4 (so that no vector straddles the matrix edge).
-  const bool vec4 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB) &&
-                    (p.a_kmajor ? p.K : p.M) % 4 == 0 && (p.b_kmajor ? p.K : p.N) % 4 == 0;
+  const bool vec_a = aligned(p.A, p.lda, p.sA, p.rA) && (p.a_kmajor ? p.K : p.M) % 4 == 0;
+  const bool vec_b = aligned(p.B, p.ldb, p.sB, p.rB) && (p.b_kmajor ? p.K : p.N) % 4 == 0;
 
   const int cus = ctx->prop.multiProcessorCount;
   auto tiles = [&](int bm, int bn) {
@@ -399,9 +466,9 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   };
   // 128x128x16 at four workgroups per CU (33 KiB of LDS and 128 VGPRs each)
   // measured fastest among BK 8/16/32 and 2..4 workgroups per CU.
-  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, a, vec4);
-  if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, a, vec4);
-  return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, a, vec4);
+  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, a, vec_a, vec_b);
+  if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, a, vec_a, vec_b);
+  return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, a, vec_a, vec_b);
 }
 
 }  // namespace phip
