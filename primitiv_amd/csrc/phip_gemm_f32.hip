@@ -12,42 +12,10 @@
 // Two LDS stages: the loads of tile t+1 are issued before the matrix
 // instructions of tile t and written to the other stage afterwards, with one
 // barrier per tile.
-#include "phip_internal.h"
+#include "phip_gemm_f32_common.h"
 
 namespace phip {
 namespace {
-
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef float float16v __attribute__((ext_vector_type(16)));
-
-constexpr int kThreads = 256;
-constexpr int kPad = 4;  // floats appended to every LDS row
-
-struct GemmArgs {
-  const float *A;
-  const float *B;
-  float *C;
-  int M, N, K;
-  long lda, ldb, ldc;
-  long sA, sB, sC;
-  long rA, rB;
-  int tiles_m, tiles_n;
-  int splits;        // workgroups that share one C tile, each taking a K range
-  int ktiles_per_r;  // ceil(K / BK)
-  int total_ktiles;  // rbatch * ktiles_per_r
-  int atomic;        // 1: add the tile into C with atomics (split K)
-  int accumulate;    // 1: C += tile, 0: C = tile (ignored when atomic)
-};
-
-// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
-// Renumber them so that one XCD receives a contiguous run of tiles.
-__device__ inline int xcd_remap(int bid, int total) {
-  constexpr int kXcds = 8;
-  const int xcd = bid % kXcds;
-  const int idx = bid / kXcds;
-  const int q = total / kXcds, rem = total % kXcds;
-  return xcd * q + (xcd < rem ? xcd : rem) + idx;
-}
 
 // The loaders below are branch-free so that the global loads of the next tile
 // can stay in flight while the matrix instructions of the current one run: a
@@ -156,66 +124,6 @@ template <int BX, int BK, int V>
 struct LoaderSelect<true, BX, BK, V> {
   typedef LoaderKContig<BX, BK, V> type;
 };
-
-// Writes NV results of one lane into C.  Result q belongs to row m and column
-// ncol + nq[q], where (m, ncol) = (row0 + lane%32, col0 + 4*(lane/32)) and nq[]
-// is the same for all lanes.  The old values of an accumulating write are
-// fetched first, all NV loads in flight together.
-//  * Interior tiles: every address is a wave-uniform base (row0, col0 + nq[q])
-//    plus one per-lane 32-bit offset, no predicates.
-//  * Edge tiles: per-element predicates; an element outside the matrix reads
-//    the matrix origin instead and is not stored.
-template <int NV>
-__device__ inline void emit_c(float *Cz, long ldc, int row0, int col0, int lane, int M, int N, bool interior,
-                              const int (&nq)[NV], const float (&vals)[NV], int atomic, int accumulate) {
-  if (interior) {
-    const unsigned voff = (unsigned)((lane & 31) + 4L * (lane >> 5) * ldc);
-    float *base[NV];
-#pragma unroll
-    for (int q = 0; q < NV; ++q) base[q] = Cz + row0 + (long)(col0 + nq[q]) * ldc;  // uniform
-    if (atomic) {
-#pragma unroll
-      for (int q = 0; q < NV; ++q) unsafeAtomicAdd(base[q] + voff, vals[q]);
-    } else if (accumulate) {
-      float old[NV];
-#pragma unroll
-      for (int q = 0; q < NV; ++q) old[q] = base[q][voff];
-#pragma unroll
-      for (int q = 0; q < NV; ++q) base[q][voff] = old[q] + vals[q];
-    } else {
-#pragma unroll
-      for (int q = 0; q < NV; ++q) base[q][voff] = vals[q];
-    }
-    return;
-  }
-  const int m = row0 + (lane & 31);
-  const int ncol = col0 + 4 * (lane >> 5);
-  constexpr int kChunk = NV < 4 ? NV : 4;  // few live addresses: this path is rare
-#pragma unroll
-  for (int c = 0; c < NV; c += kChunk) {
-    bool ok[kChunk];
-    float *p[kChunk];
-    float old[kChunk];
-#pragma unroll
-    for (int q = 0; q < kChunk; ++q) {
-      ok[q] = m < M && ncol + nq[c + q] < N;
-      p[q] = ok[q] ? Cz + m + (long)(ncol + nq[c + q]) * ldc : Cz;
-    }
-    if (atomic) {
-#pragma unroll
-      for (int q = 0; q < kChunk; ++q)
-        if (ok[q]) unsafeAtomicAdd(p[q], vals[c + q]);
-    } else {
-      if (accumulate) {
-#pragma unroll
-        for (int q = 0; q < kChunk; ++q) old[q] = *p[q];
-      }
-#pragma unroll
-      for (int q = 0; q < kChunk; ++q)
-        if (ok[q]) *p[q] = accumulate ? old[q] + vals[c + q] : vals[c + q];
-    }
-  }
-}
 
 // WGM x WGN x WGK wavefronts: WGM*WGN of them tile the BM x BN block, WGK of
 // them share each wave tile and split the k steps of every K tile between
@@ -367,19 +275,6 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_f32_kernel(const GemmArgs 
   }
 }
 
-__global__ __launch_bounds__(kThreads) void zero_c_kernel(float *C, int M, int N, long ldc, long sC, int batch) {
-  const long per = (long)M * N;
-  const long total = per * batch;
-  for (long i = (long)blockIdx.x * kThreads + threadIdx.x; i < total; i += (long)gridDim.x * kThreads) {
-    const long z = i / per, e = i - z * per;
-    C[z * sC + (e % M) + (e / M) * ldc] = 0.0f;
-  }
-}
-
-struct TileChoice {
-  int bm, bn, bk;
-};
-
 template <int BM, int BN, int BK, int WGM, int WGN, int WGK, int OCC>
 int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec_a, bool vec_b) {
   a.tiles_m = (p.M + BM - 1) / BM;
@@ -441,6 +336,9 @@ int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec_a, bool vec_b
 
 int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return PHIP_OK;
+  bool handled = false;
+  const int rc = gemm_f32_direct(ctx, p, &handled);
+  if (rc != PHIP_OK || handled) return rc;
   GemmArgs a;
   a.A = static_cast<const float *>(p.A);
   a.B = static_cast<const float *>(p.B);
