@@ -14,6 +14,8 @@
 // Global loads are raw buffer loads: everything past the end of the matrix
 // reads as zero, which covers the ragged last K tile (or the last rows) without
 // branches; the other edge is a per-lane offset select.
+#include <cstdlib>
+
 #include "phip_internal.h"
 #include "phip_types.h"
 
@@ -156,6 +158,34 @@ __device__ inline uint16_t round_c(float x) {
   else return __builtin_bit_cast(uint16_t, from_f32<f16_t>(x));
 }
 
+// Writes the 16 results one lane holds for a 32x32 block (row row0 + lane%32,
+// columns col0 + 4*(lane/32) + 8*(v/4) + v%4) into the 16-bit C.  For an
+// accumulating write the 16 old values are fetched first, all in flight
+// together; an element outside the matrix reads the matrix origin instead and
+// is not stored.
+template <bool BF16>
+__device__ inline void emit_c16(uint16_t *Cz, long ldc, int row0, int col0, int lane, int M, int N, bool interior,
+                                const float16v &acc, int accumulate) {
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+  uint16_t *p[16];
+  bool ok[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int n = ncol + 8 * (v / 4) + (v % 4);
+    ok[v] = interior || (m < M && n < N);
+    p[v] = ok[v] ? Cz + m + (long)n * ldc : Cz;
+  }
+  float old[16];
+  if (accumulate) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) old[v] = load_c<BF16>(p[v]);
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v)
+    if (ok[v]) *p[v] = round_c<BF16>(accumulate ? old[v] + acc[v] : acc[v]);
+}
+
 template <bool A_KMAJOR, bool B_KMAJOR, bool BF16>
 __global__ __launch_bounds__(kThreads, 1) void gemm_h16_big_kernel(const BigArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -263,29 +293,281 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_big_kernel(const BigArgs
   // Lane l of result register v holds C(m, n) with m = l % 32 and
   // n = 8*(v/4) + 4*(l/32) + v%4 inside its 32x32 block.
   uint16_t *Cz = g.C + (long)z * g.sC;
-  const int cm = m0 + wm * 128 + (lane & 31);
-  const int cn = n0 + wn * 128 + 4 * (lane >> 5);
+  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = cm + i * 32;
-    if (m >= g.M) continue;
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      emit_c16<BF16>(Cz, g.ldc, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32, lane, g.M, g.N, interior,
+                     acc[i][j], g.accumulate);
+}
+
+// ---------------------------------------------------------------------------
+// Second generation of the large-tile kernel: operands go from global memory
+// straight into LDS (buffer loads with the LDS destination: no registers, no
+// LDS write instructions) and an operand that is contiguous along m or n is
+// transposed by the LDS read itself (ds_read_b64_tr_b16).
+//
+// LDS image of one stage (64 KiB): A region then B region, 32 KiB each.
+//  * k-contiguous operand: 256 rows (m or n) of 64 k = 128 bytes = 8 chunks
+//    of 16 bytes.  Chunk c of row x sits at position c ^ ((x >> 1) & 7): the
+//    16 lanes of a 16-byte fragment read (consecutive rows, same c) then hit
+//    16 different 16-byte bank groups.
+//  * m/n-contiguous operand: 64 rows (k) of 256 elements = 512 bytes = 32
+//    chunks.  Chunk c of row k sits at position c ^ ((k & 3) << 2): the four k
+//    rows one transposing read touches land in different bank groups.
+// A load instruction moves 64 x 16 bytes to 1 KiB of consecutive LDS (lane l
+// to byte 16*l), so the swizzle is applied by choosing which global chunk each
+// lane fetches.
+constexpr int kRegionBytes = 32768;
+constexpr int kStage2Bytes = 2 * kRegionBytes;
+constexpr int kLds2Bytes = 2 * kStage2Bytes;
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor spelled out as four dwords (base, base high + stride 0,
+// size in bytes, format word), for use as an inline-assembly operand.
+__device__ inline uint4v make_rsrc_words(const uint16_t *p, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  uint4v r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+  return r;
+}
+
+// One 16-byte-per-lane buffer load whose destination is LDS: lane l's data
+// lands at lds_addr + 16*l.  Issued as inline assembly so that the compiler
+// does not put a wait for it in front of every later LDS read; the kernel
+// waits for these loads itself (s_waitcnt vmcnt) before the barrier that
+// publishes the tile.
+__device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "memory", "m0");
+}
+
+template <bool KMAJOR>
+struct LdsLoader {
+  uint32_t off[8];     // byte offset of this lane's chunk for each of the wave's 8 instructions, at K tile 0
+  uint32_t step;       // bytes per K tile
+  uint32_t live_mask;  // bit q: instruction q's chunk exists (along the axis that needs a predicate)
+  int kc[8];           // (k-contiguous only) first k of the chunk inside the tile, per instruction
+
+  __device__ inline void init(long ld, int x0, int X, int wave, int lane) {
+    live_mask = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int blk = wave * 8 + q;  // which 1 KiB block of the region
+      if constexpr (KMAJOR) {
+        const int x = blk * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((x >> 1) & 7);
+        off[q] = (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2);  // a row past X is past the end
+        kc[q] = c * 8;
+      } else {
+        const int k = blk * 2 + (lane >> 5);
+        const int c = (lane & 31) ^ ((k & 3) << 2);
+        off[q] = (uint32_t)(((long)k * ld + x0 + c * 8) * 2);    // a row past K is past the end
+        kc[q] = 0;
+        if (x0 + c * 8 < X) live_mask |= 1u << q;
+      }
+    }
+    step = KMAJOR ? (uint32_t)(BK * 2) : (uint32_t)(BK * ld * 2);
+  }
+
+  // Issues instruction q of K tile `kt_in_r`; `live` false makes it a no-op read.
+  __device__ inline void issue(uint4v rsrc, uint32_t region_addr, int wave, int q, int kt_in_r, int K,
+                               bool live) const {
+    bool in = live;
+    if constexpr (KMAJOR) in = in && kt_in_r * BK + kc[q] < K;
+    else in = in && ((live_mask >> q) & 1u);
+    const uint32_t o = in ? off[q] + (uint32_t)kt_in_r * step : kOutOfRange;
+    lds_dma_b128(rsrc, region_addr + (uint32_t)(wave * 8 + q) * 1024u, o);
+  }
+};
+
+// Per-lane constants of the fragment reads of one operand.
+template <bool KMAJOR>
+struct FragReader {
+  uint32_t base[4];  // byte offsets inside the region
+
+  __device__ inline void init(int xw, int lane) {
+    if constexpr (KMAJOR) {
+      // row x = xw + 32 i + lane%32, chunk (2 s + lane/32) ^ swizzle: base[s]
+      const int sw = ((lane & 31) >> 1) & 7;
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        base[s] = (uint32_t)((xw + (lane & 31)) * 128 + (((2 * s + (lane >> 5)) ^ sw) * 16));
+    } else {
+      // lane = 16 g + 4 cc + a: supplies k row cc, columns 16 (g%2) + 4 a .. +3: base[i]
+      const int h = lane >> 5, cc = (lane & 15) >> 2, a = lane & 3;
+      const int cl = (16 * ((lane >> 4) & 1) + 4 * a) >> 3;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        base[i] = (uint32_t)((8 * h + cc) * 512 + (xw / 8 + 4 * (i ^ cc) + cl) * 16 + (a & 1) * 8);
+    }
+  }
+
+  // Fragment of 32x32 block i for k step s: 8 consecutive k of row lane%32.
+  __device__ inline uint4v read(const unsigned char *region, int i, int s) const {
+    if constexpr (KMAJOR) {
+      return *reinterpret_cast<const uint4v *>(region + base[s] + i * 4096);
+    } else {
+      const unsigned char *p = region + base[i] + s * 16 * 512;
+      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) short4v *)(p));
+      const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) short4v *)(p + 4 * 512));
+      uint4v r;
+      r.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+      r.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+      r.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+      r.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+      return r;
+    }
+  }
+};
+
+template <bool A_KMAJOR, bool B_KMAJOR, bool BF16>
+__global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+
+  int t = xcd_remap(blockIdx.x, gridDim.x);
+  const int per_z = g.tiles_m * g.tiles_n;
+  const int z = t / per_z;
+  t -= z * per_z;
+  constexpr int GM = 8;
+  const int group = t / (GM * g.tiles_n);
+  const int first_m = group * GM;
+  const int gm = g.tiles_m - first_m < GM ? g.tiles_m - first_m : GM;
+  const int in_group = t - group * GM * g.tiles_n;
+  const int tile_m = first_m + in_group % gm;
+  const int tile_n = in_group / gm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  LdsLoader<A_KMAJOR> la;
+  LdsLoader<B_KMAJOR> lb;
+  la.init(g.lda, m0, g.M, wave, lane);
+  lb.init(g.ldb, n0, g.N, wave, lane);
+  FragReader<A_KMAJOR> fra;
+  FragReader<B_KMAJOR> frb;
+  fra.init(wm * 128, lane);
+  frb.init(wn * 128, lane);
+
+  const uint16_t *Az = g.A + (long)z * g.sA;
+  const uint16_t *Bz = g.B + (long)z * g.sB;
+
+  float16v acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
-        if (n < g.N) {
-          uint16_t *p = Cz + m + (long)n * g.ldc;
-          const float s = acc[i][j][v];
-          *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int kt_end = g.total_ktiles;
+  // Every workgroup starts its walk over K at a different tile (and wraps
+  // around): with power-of-two leading dimensions, workgroups marching through
+  // K in lockstep would all pull from the same memory channels at once.
+  const int kt_rot = (tile_m + tile_n + z) % kt_end;
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds2;
+  auto issue_tile = [&](int kt, int q_first, int q_count) {
+    // instructions [q_first, q_first + q_count) of the 16 that move K tile kt (8 for A, then 8 for B)
+    const bool live = kt < kt_end;
+    int ktc = live ? kt + kt_rot : 0;
+    ktc = ktc >= kt_end ? ktc - kt_end : ktc;
+    const int r = ktc / g.ktiles_per_r;
+    const int kt_in_r = ktc - r * g.ktiles_per_r;
+    const uint32_t stage = lds_base + (uint32_t)(kt & 1) * kStage2Bytes;
+#pragma unroll
+    for (int q = q_first; q < q_first + q_count; ++q) {
+      if (q < 8) la.issue(make_rsrc_words(Az + (long)r * g.rA, g.a_bytes), stage, wave, q, kt_in_r, g.K, live);
+      else lb.issue(make_rsrc_words(Bz + (long)r * g.rB, g.b_bytes), stage + kRegionBytes, wave, q - 8, kt_in_r,
+                    g.K, live);
+    }
+  };
+
+  issue_tile(0, 0, 16);
+  issue_tile(1, 0, 16);
+  // tile 0 has landed once all but the newest 16 loads are done
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  __syncthreads();
+
+  uint4v fa[2][4], fb[2][4];
+  auto read_frag = [&](int buf, int q, int stage, int s) {
+    const unsigned char *st = lds2 + stage * kStage2Bytes;
+    if (q < 4) fa[buf][q] = fra.read(st, q, s);
+    else fb[buf][q - 4] = frb.read(st + kRegionBytes, q - 4, s);
+  };
+#pragma unroll
+  for (int q = 0; q < 8; ++q) read_frag(0, q, 0, 0);
+
+  for (int kt = 0; kt < kt_end; ++kt) {
+    const int stage = kt & 1;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int cur = s & 1, nxt = cur ^ 1;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int i = q >> 2, j = q & 3;
+        acc[i][j] = mfma<BF16>(fb[cur][j], fa[cur][i], acc[i][j]);
+        if (q < 8) {
+          if (s < 3) read_frag(nxt, q, stage, s + 1);
+          else read_frag(nxt, q, stage ^ 1, 0);
         }
+        // K tile kt+2 refills this stage once everybody has left it
+        if (s == 3) issue_tile(kt + 2, q, 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      if (s == 2) {
+        // own loads of tile kt+1 have landed, own reads of this stage are done;
+        // behind the barrier that holds for every wave
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+      }
+    }
   }
+  // the loads issued for tiles past the end move nothing, but must have retired
+  // before this workgroup's LDS can be handed to another one
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  uint16_t *Cz = g.C + (long)z * g.sC;
+  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      emit_c16<BF16>(Cz, g.ldc, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32, lane, g.M, g.N, interior,
+                     acc[i][j], g.accumulate);
 }
 
 template <bool BF16>
 int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
   const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
+  static const bool use_v1 = getenv("PHIP_H16_V1") != nullptr;
+  if (!use_v1) {
+#define PHIP_LDS(AK, BKM)                                                                        \
+  do {                                                                                           \
+    auto kern = gemm_h16_lds_kernel<AK, BKM, BF16>;                                              \
+    static bool configured = false;                                                              \
+    if (!configured) {                                                                           \
+      PHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                         \
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLds2Bytes));     \
+      configured = true;                                                                         \
+    }                                                                                            \
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLds2Bytes, ctx->stream, a);  \
+  } while (0)
+    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(false, true);
+    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(false, false);
+    else if (p.a_kmajor && p.b_kmajor) PHIP_LDS(true, true);
+    else return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
+#undef PHIP_LDS
+    PHIP_LAUNCH_CHECK();
+    return PHIP_OK;
+  }
 #define PHIP_BIG(AK, BKM)                                                                        \
   do {                                                                                           \
     auto kern = gemm_h16_big_kernel<AK, BKM, BF16>;                                              \
