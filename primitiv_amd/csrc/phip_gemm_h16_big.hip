@@ -1,21 +1,19 @@
 // Large-tile GEMM for 16-bit storage (fp16 / bf16, fp32 accumulation):
 // 256 x 256 x 64 tiles, one workgroup (4 wavefronts, each a 128 x 128 block of
-// 4 x 4 v_mfma_f32_32x32x16 tiles) per CU, two 72 KiB LDS stages.
+// 4 x 4 v_mfma_f32_32x32x16 tiles, 256 accumulator registers per lane) per CU,
+// two 64 KiB LDS stages.
 //
-// LDS holds both operands as rows of 64 consecutive k (+8 elements of padding):
-// the matrix instruction takes 8 consecutive k per lane, so every fragment is
-// one 16-byte LDS read, conflict-free with the 144-byte row stride.
-//  * An operand that is contiguous along k in memory is copied: 8 lanes read
-//    one 128-byte line of a row and write it to the LDS row.
-//  * An operand that is contiguous along m or n is transposed in registers:
-//    a thread loads an 8 (k) x 8 (m) block as eight 16-byte rows, transposes
-//    it with 32 byte-permutes and writes eight 16-byte LDS rows; 8 lanes
-//    again cover 128 contiguous bytes on both sides.
-// Global loads are raw buffer loads: everything past the end of the matrix
-// reads as zero, which covers the ragged last K tile (or the last rows) without
-// branches; the other edge is a per-lane offset select.
-#include <cstdlib>
-
+// Nothing is staged through registers and nothing is transposed by ALU work:
+//  * both operands are moved global -> LDS by buffer loads that write LDS
+//    directly; everything past the end of a matrix reads as zero (buffer range
+//    check), which covers ragged edges without branches;
+//  * an operand that is contiguous along k is read back with 16-byte LDS reads
+//    (8 consecutive k per lane is what the matrix instruction takes);
+//  * an operand that is contiguous along m or n is kept in LDS as it is in
+//    memory and transposed by the LDS read instruction (ds_read_b64_tr_b16).
+// LDS rows are not padded (a load instruction fills 1 KiB of consecutive LDS);
+// bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row
+// each lane fetches.
 #include "phip_internal.h"
 #include "phip_types.h"
 
@@ -29,9 +27,6 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int S = BK + 8;                       // LDS row stride in elements
-constexpr int kStageA = BM * S, kStageB = BN * S;
-constexpr int kLdsBytes = 2 * (kStageA + kStageB) * 2;
 constexpr uint32_t kOutOfRange = 0x80000000u;   // beyond any buffer this kernel accepts
 
 struct BigArgs {
@@ -56,83 +51,6 @@ __device__ inline int xcd_remap(int bid, int total) {
   const int q = total / kXcds, rem = total % kXcds;
   return xcd * q + (xcd < rem ? xcd : rem) + idx;
 }
-
-__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const uint16_t *p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p), 0, (int)bytes, 0x00020000);
-}
-
-// One operand's 256 x 64 tile.  KMAJOR: element (x, k) at k + x*ld.
-// Otherwise: element (x, k) at x + k*ld.
-template <bool KMAJOR>
-struct TileLoader {
-  uint4v regs[8];
-  uint32_t off[8];   // byte offsets of this thread's eight vectors at k0 = 0
-  uint32_t step;     // bytes to advance per K tile
-  int kg;            // which 8-wide k group of the tile this thread serves
-  bool x_in;         // (x-contiguous only) the thread's 8 columns exist
-  uint32_t lds_off;  // element offset of this thread's first LDS row segment
-
-  __device__ inline void init(long ld, int x0, int X, int tid) {
-    kg = tid & 7;
-    const int xr = tid >> 3;
-    if constexpr (KMAJOR) {
-      // rows x = x0 + xr + 32 i; a row past X starts past the end of the matrix
-#pragma unroll
-      for (int i = 0; i < 8; ++i) off[i] = (uint32_t)(((long)(x0 + xr + 32 * i) * ld + kg * 8) * 2);
-      step = BK * 2;
-      x_in = true;
-      lds_off = xr * S + kg * 8;
-    } else {
-      // an 8 x 8 block: k rows kg*8 + i, columns x0 + xr*8 .. +7
-#pragma unroll
-      for (int i = 0; i < 8; ++i) off[i] = (uint32_t)(((long)(kg * 8 + i) * ld + x0 + xr * 8) * 2);
-      step = (uint32_t)(BK * ld * 2);
-      x_in = x0 + xr * 8 < X;
-      lds_off = (xr * 8) * S + kg * 8;
-    }
-  }
-
-  // Prepares tile `kt_in_r` of the current sample; `live` false turns every
-  // load of the tile into an out-of-range one (reads zeros, touches nothing).
-  uint32_t adv;
-  bool in;
-  __device__ inline void begin(int kt_in_r, int K, bool live) {
-    adv = (uint32_t)kt_in_r * step;
-    if constexpr (KMAJOR) in = live && kt_in_r * BK + kg * 8 < K;  // the next column starts right after K
-    else in = live && x_in;                                         // rows past K are past the end
-  }
-  __device__ inline void load_one(__amdgpu_buffer_rsrc_t rsrc, int i) {
-    const uint32_t o = in ? off[i] + adv : kOutOfRange;
-    regs[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)o, 0, 0);
-  }
-  __device__ inline void load(__amdgpu_buffer_rsrc_t rsrc, int kt_in_r, int K) {
-    begin(kt_in_r, K, true);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) load_one(rsrc, i);
-  }
-
-  // Writes the j-th of this thread's eight 16-byte LDS row segments.
-  __device__ inline void store_one(uint16_t *lds, int j) const {
-    uint16_t *p = lds + lds_off;
-    if constexpr (KMAJOR) {
-      *reinterpret_cast<uint4v *>(p + 32 * j * S) = regs[j];
-    } else {
-      // regs[i] = 8 columns of k row i.  Output row j = column j across the 8
-      // k rows: dword d of it packs (row 2d, row 2d+1) of element j.
-      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-      uint4v o;
-      o.x = __builtin_amdgcn_perm(regs[1][j >> 1], regs[0][j >> 1], sel);
-      o.y = __builtin_amdgcn_perm(regs[3][j >> 1], regs[2][j >> 1], sel);
-      o.z = __builtin_amdgcn_perm(regs[5][j >> 1], regs[4][j >> 1], sel);
-      o.w = __builtin_amdgcn_perm(regs[7][j >> 1], regs[6][j >> 1], sel);
-      *reinterpret_cast<uint4v *>(p + j * S) = o;
-    }
-  }
-  __device__ inline void store(uint16_t *lds) const {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) store_one(lds, j);
-  }
-};
 
 template <bool BF16>
 __device__ inline float16v mfma(uint4v a, uint4v b, float16v c) {
@@ -186,127 +104,11 @@ __device__ inline void emit_c16(uint16_t *Cz, long ldc, int row0, int col0, int 
     if (ok[v]) *p[v] = round_c<BF16>(accumulate ? old[v] + acc[v] : acc[v]);
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, bool BF16>
-__global__ __launch_bounds__(kThreads, 1) void gemm_h16_big_kernel(const BigArgs g) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;
-
-  // Tile order: z slowest; inside one sample, groups of 8 tile rows are walked
-  // column by column so that the ~32 tiles an XCD runs together share panels.
-  int t = xcd_remap(blockIdx.x, gridDim.x);
-  const int per_z = g.tiles_m * g.tiles_n;
-  const int z = t / per_z;
-  t -= z * per_z;
-  constexpr int GM = 8;
-  const int group = t / (GM * g.tiles_n);
-  const int first_m = group * GM;
-  const int gm = g.tiles_m - first_m < GM ? g.tiles_m - first_m : GM;
-  const int in_group = t - group * GM * g.tiles_n;
-  const int tile_m = first_m + in_group % gm;
-  const int tile_n = in_group / gm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-  TileLoader<A_KMAJOR> la;
-  TileLoader<B_KMAJOR> lb;
-  la.init(g.lda, m0, g.M, tid);
-  lb.init(g.ldb, n0, g.N, tid);
-
-  const uint16_t *Az = g.A + (long)z * g.sA;
-  const uint16_t *Bz = g.B + (long)z * g.sB;
-
-  float16v acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  const int kt_end = g.total_ktiles;
-  {
-    la.load(make_rsrc(Az, g.a_bytes), 0, g.K);
-    lb.load(make_rsrc(Bz, g.b_bytes), 0, g.K);
-    la.store(lds);
-    lb.store(lds + 2 * kStageA);
-  }
-  __syncthreads();
-
-  // Lane l supplies row l%32 and the 8 k values starting at 8*(l/32).
-  const int frag_off = (lane & 31) * S + 8 * (lane >> 5);
-  const uint16_t *a_frag = lds + wm * 128 * S + frag_off;
-  const uint16_t *b_frag = lds + 2 * kStageA + wn * 128 * S + frag_off;
-
-  // Fragments are double-buffered in registers: the reads of k step s+1 are
-  // issued between the matrix instructions of step s, and the first step of
-  // the next tile is read behind the barrier, under the last step of this one.
-  uint4v fa[2][4], fb[2][4];
-  auto read_frag = [&](int buf, int q, int stage, int s) {
-    if (q < 4) fa[buf][q] = *reinterpret_cast<const uint4v *>(a_frag + stage * kStageA + q * 32 * S + s * 16);
-    else fb[buf][q - 4] = *reinterpret_cast<const uint4v *>(b_frag + stage * kStageB + (q - 4) * 32 * S + s * 16);
-  };
-#pragma unroll
-  for (int q = 0; q < 8; ++q) read_frag(0, q, 0, 0);
-
-  for (int kt = 0; kt < kt_end; ++kt) {
-    const int stage = kt & 1;
-    // Next tile (loads degenerate to out-of-range reads after the last one).
-    const bool more = kt + 1 < kt_end;
-    const int nkt = more ? kt + 1 : kt;
-    const int r = nkt / g.ktiles_per_r;
-    const int kt_in_r = nkt - r * g.ktiles_per_r;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Az + (long)r * g.rA, g.a_bytes);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bz + (long)r * g.rB, g.b_bytes);
-    la.begin(kt_in_r, g.K, more);
-    lb.begin(kt_in_r, g.K, more);
-    uint16_t *next_a = lds + (stage ^ 1) * kStageA;
-    uint16_t *next_b = lds + 2 * kStageA + (stage ^ 1) * kStageB;
-
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int cur = s & 1, nxt = cur ^ 1;
-#pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const int i = q >> 2, j = q & 3;
-        acc[i][j] = mfma<BF16>(fb[cur][j], fa[cur][i], acc[i][j]);
-        // work slotted in behind this matrix instruction
-        if (s == 0) {
-          if (q < 8) la.load_one(ra, q); else lb.load_one(rb, q - 8);
-        }
-        if (q < 8) {
-          if (s < 3) read_frag(nxt, q, stage, s + 1);
-          else read_frag(nxt, q, stage ^ 1, 0);
-        }
-        if (s == 2) {
-          if (q < 8) la.store_one(next_a, q); else lb.store_one(next_b, q - 8);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (s == 2) __syncthreads();
-    }
-  }
-
-  // Lane l of result register v holds C(m, n) with m = l % 32 and
-  // n = 8*(v/4) + 4*(l/32) + v%4 inside its 32x32 block.
-  uint16_t *Cz = g.C + (long)z * g.sC;
-  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      emit_c16<BF16>(Cz, g.ldc, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32, lane, g.M, g.N, interior,
-                     acc[i][j], g.accumulate);
-}
-
 // ---------------------------------------------------------------------------
-// Second generation of the large-tile kernel: operands go from global memory
-// straight into LDS (buffer loads with the LDS destination: no registers, no
-// LDS write instructions) and an operand that is contiguous along m or n is
-// transposed by the LDS read itself (ds_read_b64_tr_b16).
+// Operands go from global memory straight into LDS (buffer loads with the LDS
+// destination: no registers, no LDS write instructions) and an operand that
+// is contiguous along m or n is transposed by the LDS read itself
+// (ds_read_b64_tr_b16).
 //
 // LDS image of one stage (64 KiB): A region then B region, 32 KiB each.
 //  * k-contiguous operand: 256 rows (m or n) of 64 k = 128 bytes = 8 chunks
@@ -342,7 +144,7 @@ __device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t vof
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                :
                : "s"(lds_addr), "v"(voffset), "s"(rsrc)
-               : "memory", "m0");
+               : "memory");  // m0 is scratch between instructions: nothing else in this kernel keeps a value in it
 }
 
 template <bool KMAJOR>
@@ -496,7 +298,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs
   asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   __syncthreads();
 
-  uint4v fa[2][4], fb[2][4];
+  // Fragments of the four k steps of a tile live in four register buffers and
+  // are read two steps ahead: steps 2 and 3 of this tile during steps 0 and 1,
+  // then - behind the barrier - steps 0 and 1 of the next tile during steps 2
+  // and 3.  The barrier therefore sits in the middle of a tile, and the
+  // global-to-LDS loads that refill the stage (K tile kt+2) are spread over
+  // the 32 instruction slots of steps 2 and 3, with a whole tile time to land.
+  uint4v fa[4][4], fb[4][4];
   auto read_frag = [&](int buf, int q, int stage, int s) {
     const unsigned char *st = lds2 + stage * kStage2Bytes;
     if (q < 4) fa[buf][q] = fra.read(st, q, s);
@@ -504,25 +312,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs
   };
 #pragma unroll
   for (int q = 0; q < 8; ++q) read_frag(0, q, 0, 0);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) read_frag(1, q, 0, 1);
 
   for (int kt = 0; kt < kt_end; ++kt) {
     const int stage = kt & 1;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int cur = s & 1, nxt = cur ^ 1;
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int i = q >> 2, j = q & 3;
-        acc[i][j] = mfma<BF16>(fb[cur][j], fa[cur][i], acc[i][j]);
+        acc[i][j] = mfma<BF16>(fb[s][j], fa[s][i], acc[i][j]);
         if (q < 8) {
-          if (s < 3) read_frag(nxt, q, stage, s + 1);
-          else read_frag(nxt, q, stage ^ 1, 0);
+          if (s < 2) read_frag(s + 2, q, stage, s + 2);
+          else read_frag(s - 2, q, stage ^ 1, s - 2);
         }
-        // K tile kt+2 refills this stage once everybody has left it
-        if (s == 3) issue_tile(kt + 2, q, 1);
+        if (s >= 2 && (q & 1)) issue_tile(kt + 2, (s - 2) * 8 + (q >> 1), 1);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 2) {
+      if (s == 1) {
         // own loads of tile kt+1 have landed, own reads of this stage are done;
         // behind the barrier that holds for every wave
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -547,8 +355,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs
 template <bool BF16>
 int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
   const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
-  static const bool use_v1 = getenv("PHIP_H16_V1") != nullptr;
-  if (!use_v1) {
 #define PHIP_LDS(AK, BKM)                                                                        \
   do {                                                                                           \
     auto kern = gemm_h16_lds_kernel<AK, BKM, BF16>;                                              \
@@ -560,30 +366,11 @@ int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
     }                                                                                            \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLds2Bytes, ctx->stream, a);  \
   } while (0)
-    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(false, true);
-    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(false, false);
-    else if (p.a_kmajor && p.b_kmajor) PHIP_LDS(true, true);
-    else return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
-#undef PHIP_LDS
-    PHIP_LAUNCH_CHECK();
-    return PHIP_OK;
-  }
-#define PHIP_BIG(AK, BKM)                                                                        \
-  do {                                                                                           \
-    auto kern = gemm_h16_big_kernel<AK, BKM, BF16>;                                              \
-    static bool configured = false;                                                              \
-    if (!configured) {                                                                           \
-      PHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                         \
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));      \
-      configured = true;                                                                         \
-    }                                                                                            \
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, ctx->stream, a);   \
-  } while (0)
-  if (!p.a_kmajor && p.b_kmajor) PHIP_BIG(false, true);
-  else if (!p.a_kmajor && !p.b_kmajor) PHIP_BIG(false, false);
-  else if (p.a_kmajor && p.b_kmajor) PHIP_BIG(true, true);
+  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(false, true);
+  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(false, false);
+  else if (p.a_kmajor && p.b_kmajor) PHIP_LDS(true, true);
   else return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
-#undef PHIP_BIG
+#undef PHIP_LDS
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
 }
