@@ -364,7 +364,10 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   };
   // 128x128x16 at four workgroups per CU (33 KiB of LDS and 128 VGPRs each)
   // measured fastest among BK 8/16/32 and 2..4 workgroups per CU.
-  if (tiles(128, 128) >= cus) return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, a, vec_a, vec_b);
+  // A short contraction (K <= 128) is a rank-K update bound by the traffic of
+  // C and by latency: 64x64 tiles put four times as many workgroups in flight.
+  const long k_total = (long)p.K * p.rbatch;
+  if (tiles(128, 128) >= cus && k_total > 128) return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, a, vec_a, vec_b);
   if (tiles(64, 64) >= cus) return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, a, vec_a, vec_b);
   return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, a, vec_a, vec_b);
 }

@@ -247,12 +247,13 @@ int gemm_f32_direct(phip_ctx *ctx, const Gemm &p, bool *handled) {
   const bool wide = p.N > 32 && tiles(32, 64) * 2 >= cus;
   const long t = wide ? tiles(32, 64) : tiles(32, 32);
   // Split K between workgroups until about two workgroups per CU are busy,
-  // keeping at least 8 chunks (64 k) per wavefront.  An overwriting product
+  // keeping at least 4 chunks (32 k) per wavefront (measured best on the
+  // recurrent-gate and output-projection gradients).  An overwriting product
   // is only split when it would otherwise leave most of the chip idle: the
   // split needs a zero fill of C in front of it.
   int splits = 1;
   const long want = (2L * cus + t - 1) / t;
-  long cap = d.total_chunks / 32;
+  long cap = d.total_chunks / 16;
   if (cap < 1) cap = 1;
   if (p.accumulate || t * 8 <= cus) splits = (int)(want < cap ? want : cap);
   if (splits < 1) splits = 1;
