@@ -101,7 +101,7 @@ __device__ inline void emit_c(float *Cz, long ldc, int row0, int col0, int lane,
   }
 }
 
-__global__ __launch_bounds__(kThreads) void zero_c_kernel(float *C, int M, int N, long ldc, long sC, int batch) {
+__attribute__((unused)) __global__ __launch_bounds__(kThreads) void zero_c_kernel(float *C, int M, int N, long ldc, long sC, int batch) {
   const long per = (long)M * N;
   const long total = per * batch;
   for (long i = (long)blockIdx.x * kThreads + threadIdx.x; i < total; i += (long)gridDim.x * kThreads) {

@@ -183,6 +183,33 @@ def test_random_shapes_h16(dev16, devbf16, which, ba, bb):
                 assert norm_rel_err(got, ref) <= tol, name + " " + tag
 
 
+# shapes that reach the fp32 128x128x32 global-to-LDS kernel (>= one tile per CU)
+# with ragged edges in every dimension (multiples of 4, not of 128 / 32)
+BIG_F32 = [  # di, dj, dk, ba, bb
+    (2056, 2064, 2072, 1, 1),
+    (776, 520, 1032, 16, 16),
+    (136, 2056, 2064, 16, 1),
+    (2056, 264, 520, 1, 4),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", BIG_F32)
+def test_large_tile_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di + dj + dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    y, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(y, ry) <= F32_TOL
+    assert norm_rel_err(ga, rga) <= F32_TOL
+    assert norm_rel_err(gb, rgb) <= F32_TOL
+
+
 # shapes that reach the 256x256x64 large-tile kernel with ragged edges in every
 # dimension (multiples of 8, not of 256 / 64), in each batch case
 BIG_H16 = [  # di, dj, dk, ba, bb
