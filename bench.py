@@ -33,7 +33,7 @@ HEADLINE = "square_batched"
 # HBM bytes per launch of the headline kernel (average of its three operand-layout
 # instantiations): rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors read
 # off a streaming y += x of known size (the summary under profiles/ holds both runs).
-HEADLINE_TRAFFIC_BYTES = 220.2e6 + 73.4e6
+HEADLINE_TRAFFIC_BYTES = 195.9e6 + 67.1e6
 
 
 class Resident:
@@ -184,16 +184,17 @@ def main():
 
     head = results.get(HEADLINE) or results[names[0]]
     w = WORKLOADS[head["workload"]]
-    # Dominant kernel of the headline workload: the 128x128x16 fp32 MFMA GEMM
-    # (three operand-layout instantiations, one launch each per step, equal
-    # flops); its average launch duration is the event time over the launches.
+    # Dominant kernel of the headline workload: the 128x128x32 fp32 MFMA GEMM
+    # with global-to-LDS loads (three operand-layout instantiations, one launch
+    # each per step, equal flops); its average launch duration is the event
+    # time over the launches.
     launch_s = head["ms_per_step"] * 1e-3 / (3 * w.steps)
     flops_per_launch = w.flops_per_step() / 3
     roofline = {
         "bound": "mfma", "achieved": flops_per_launch / launch_s / 1e12, "peak": PEAK_TFLOPS[w.storage],
         "unit": "TFLOP/s", "frac": flops_per_launch / launch_s / 1e12 / PEAK_TFLOPS[w.storage],
         "traffic": HEADLINE_TRAFFIC_BYTES if head["workload"] == HEADLINE else None,
-        "kernel": "gemm_f32_kernel<128,128,16,...> (fw NN, gA NT, gB TN)",
+        "kernel": "gemm_f32_lds_kernel<A_KMAJOR,B_KMAJOR> (fw, ga, gb)",
         "flops_per_launch": flops_per_launch, "avg_launch_ms": launch_s * 1e3,
     }
     line = {
