@@ -287,20 +287,16 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
 
-#define PHIP_LDS(AK, BKM)                                                                       \
+#define PHIP_LDS(SLOT, AK, BKM)                                                                 \
   do {                                                                                          \
     auto kern = gemm_f32_lds_kernel<AK, BKM>;                                                   \
-    static bool configured = false;                                                             \
-    if (!configured) {                                                                          \
-      PHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                        \
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));     \
-      configured = true;                                                                        \
-    }                                                                                           \
+    const int rc = raise_lds_limit(ctx, SLOT, reinterpret_cast<const void *>(kern), kLdsBytes); \
+    if (rc != PHIP_OK) return rc;                                                               \
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), kLdsBytes, ctx->stream, d); \
   } while (0)
-  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(false, true);
-  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(false, false);
-  else PHIP_LDS(true, true);
+  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(0, false, true);
+  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(1, false, false);
+  else PHIP_LDS(2, true, true);
 #undef PHIP_LDS
   PHIP_LAUNCH_CHECK();
   *handled = true;

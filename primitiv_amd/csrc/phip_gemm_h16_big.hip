@@ -62,46 +62,80 @@ __device__ inline float16v mfma(uint4v a, uint4v b, float16v c) {
 }
 
 template <bool BF16>
-__device__ inline float load_c(const uint16_t *p) {
-  if constexpr (BF16) {
-    bf16_t t; t.bits = *p; return to_f32(t);
-  } else {
-    return to_f32(__builtin_bit_cast(f16_t, *p));
-  }
+__device__ inline float widen(uint32_t bits16) {
+  if constexpr (BF16) return __builtin_bit_cast(float, bits16 << 16);
+  else return to_f32(__builtin_bit_cast(f16_t, (uint16_t)bits16));
 }
 
 template <bool BF16>
-__device__ inline uint16_t round_c(float x) {
+__device__ inline uint32_t round_c(float x) {
   if constexpr (BF16) return from_f32<bf16_t>(x).bits;
   else return __builtin_bit_cast(uint16_t, from_f32<f16_t>(x));
 }
 
-// Writes the 16 results one lane holds for a 32x32 block (row row0 + lane%32,
-// columns col0 + 4*(lane/32) + 8*(v/4) + v%4) into the 16-bit C.  For an
-// accumulating write the 16 old values are fetched first, all in flight
-// together; an element outside the matrix reads the matrix origin instead and
-// is not stored.
+// Writes the 128 x 128 block of results one wavefront holds into the 16-bit C,
+// 16 bytes (8 consecutive rows of one column) per lane and store instruction.
+// The matrix instruction leaves a lane with one row and 16 columns of each
+// 32 x 32 block, so the block is turned through a 32 KiB LDS area that belongs
+// to this wavefront alone: written as fp32 the way the accumulators lie,
+// read back 8 consecutive rows at a time, in two halves of 64 columns.  For an
+// accumulating write the old values are fetched (also 16 bytes per lane)
+// before the LDS pass, added in fp32 and rounded once.  M is a multiple of 8
+// and C is 16-byte aligned (checked by the dispatcher), so a lane's 8 rows are
+// either all inside the matrix or all outside.
 template <bool BF16>
-__device__ inline void emit_c16(uint16_t *Cz, long ldc, int row0, int col0, int lane, int M, int N, bool interior,
-                                const float16v &acc, int accumulate) {
-  const int m = row0 + (lane & 31);
-  const int ncol = col0 + 4 * (lane >> 5);
-  uint16_t *p[16];
-  bool ok[16];
+__device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, int row0, int col0, int lane, int M,
+                                          int N, const float16v (&acc)[4][4], int accumulate) {
+  const int mc = lane & 15, cq = lane >> 4;
+  const int m = row0 + 8 * mc;
+  // lanes 8..15 of each group of 16 read their two 16-byte halves in the other
+  // order, which spreads a 16-lane read over all banks
+  const bool flip = (mc & 8) != 0;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int n = ncol + 8 * (v / 4) + (v % 4);
-    ok[v] = interior || (m < M && n < N);
-    p[v] = ok[v] ? Cz + m + (long)n * ldc : Cz;
+  for (int h = 0; h < 2; ++h) {
+    uint16_t *p[16];
+    uint32_t ok = 0;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int n = col0 + 64 * h + 4 * it + cq;
+      const bool in = m < M && n < N;
+      ok |= (in ? 1u : 0u) << it;
+      p[it] = in ? Cz + m + (long)n * ldc : Cz;   // outside: read the origin, store nothing
+    }
+    uint4v old[16];
+    if (accumulate) {
+#pragma unroll
+      for (int it = 0; it < 16; ++it) old[it] = *reinterpret_cast<const uint4v *>(p[it]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int jl = 0; jl < 2; ++jl)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          area[(32 * jl + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4)) * 128 + 32 * i + (lane & 31)] =
+              acc[i][2 * h + jl][v];
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const float4 *src = reinterpret_cast<const float4 *>(area + (4 * it + cq) * 128 + 8 * mc);
+      const float4 first = src[flip ? 1 : 0];
+      const float4 second = src[flip ? 0 : 1];
+      const float4 lo = flip ? second : first;
+      const float4 hi = flip ? first : second;
+      float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      uint4v out;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float x0 = f[2 * e], x1 = f[2 * e + 1];
+        if (accumulate) {
+          x0 += widen<BF16>(old[it][e] & 0xffffu);
+          x1 += widen<BF16>(old[it][e] >> 16);
+        }
+        out[e] = round_c<BF16>(x0) | (round_c<BF16>(x1) << 16);
+      }
+      if ((ok >> it) & 1u) *reinterpret_cast<uint4v *>(p[it]) = out;
+    }
   }
-  float old[16];
-  if (accumulate) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) old[v] = load_c<BF16>(p[v]);
-  }
-#pragma unroll
-  for (int v = 0; v < 16; ++v)
-    if (ok[v]) *p[v] = round_c<BF16>(accumulate ? old[v] + acc[v] : acc[v]);
 }
 
 // ---------------------------------------------------------------------------
@@ -338,37 +372,30 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs
       }
     }
   }
-  // the loads issued for tiles past the end move nothing, but must have retired
-  // before this workgroup's LDS can be handed to another one
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // The loads issued for tiles past the end move nothing, but must have retired,
+  // and every wave must be done with the stages, before LDS is reused below.
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
 
   uint16_t *Cz = g.C + (long)z * g.sC;
-  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      emit_c16<BF16>(Cz, g.ldc, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32, lane, g.M, g.N, interior,
-                     acc[i][j], g.accumulate);
+  emit_block_via_lds<BF16>(reinterpret_cast<float *>(lds2 + wave * kRegionBytes), Cz, g.ldc, m0 + wm * 128,
+                           n0 + wn * 128, lane, g.M, g.N, acc, g.accumulate);
 }
 
 template <bool BF16>
 int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
   const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
-#define PHIP_LDS(AK, BKM)                                                                        \
+#define PHIP_LDS(SLOT, AK, BKM)                                                                  \
   do {                                                                                           \
     auto kern = gemm_h16_lds_kernel<AK, BKM, BF16>;                                              \
-    static bool configured = false;                                                              \
-    if (!configured) {                                                                           \
-      PHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                         \
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLds2Bytes));     \
-      configured = true;                                                                         \
-    }                                                                                            \
+    const int rc = raise_lds_limit(ctx, (SLOT) + (BF16 ? 3 : 0) + 8,                             \
+                                   reinterpret_cast<const void *>(kern), kLds2Bytes);            \
+    if (rc != PHIP_OK) return rc;                                                                \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLds2Bytes, ctx->stream, a);  \
   } while (0)
-  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(false, true);
-  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(false, false);
-  else if (p.a_kmajor && p.b_kmajor) PHIP_LDS(true, true);
+  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(0, false, true);
+  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(1, false, false);
+  else if (p.a_kmajor && p.b_kmajor) PHIP_LDS(2, true, true);
   else return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
 #undef PHIP_LDS
   PHIP_LAUNCH_CHECK();
@@ -386,6 +413,8 @@ int gemm_h16_big(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   };
   if (!aligned(p.A, p.lda, p.sA, p.rA) || !aligned(p.B, p.ldb, p.sB, p.rB)) return PHIP_OK;
   if ((p.a_kmajor ? p.K : p.M) % 8 != 0 || (p.b_kmajor ? p.K : p.N) % 8 != 0) return PHIP_OK;
+  // C is written 8 rows (16 bytes) at a time
+  if (!aligned(p.C, p.ldc, p.sC, 0) || p.M % 8 != 0) return PHIP_OK;
   // the contiguous extent of a dense operand is its leading dimension
   if ((p.a_kmajor ? p.K : p.M) != p.lda || (p.b_kmajor ? p.K : p.N) != p.ldb) return PHIP_OK;
   const long a_bytes = 2L * p.M * p.K, b_bytes = 2L * p.N * p.K;

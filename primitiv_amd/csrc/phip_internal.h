@@ -34,6 +34,9 @@ struct phip_ctx {
   hipDeviceProp_t prop;
   phip::Pool pool;
   std::mutex mutex;  // guards `pool`
+  // Kernels whose dynamic-LDS limit has been raised on this context's device
+  // (one bit per kernel, see phip::raise_lds_limit).
+  uint32_t lds_limit_raised = 0;
 };
 
 struct phip_event {
@@ -67,6 +70,15 @@ struct phip_event {
 #define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
 
 namespace phip {
+
+// Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on
+// the context's device; done once per context and kernel (`slot` < 32).
+inline int raise_lds_limit(phip_ctx *ctx, int slot, const void *kernel, int bytes) {
+  if (ctx->lds_limit_raised & (1u << slot)) return PHIP_OK;
+  PHIP_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  ctx->lds_limit_raised |= 1u << slot;
+  return PHIP_OK;
+}
 
 // ---- GEMM layer (phip_gemm_*.hip) ------------------------------------------
 //
