@@ -175,6 +175,143 @@ int phip_matmul_bw_bf16(phip_ctx *ctx, const void *a, const void *b, const void 
                         void *ga, void *gb,
                         uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
 
+/* ---- elementwise operations around the matmul ------------------------------
+ * The layers of every primitiv example wrap the matmul in a bias add and an
+ * activation (examples/mnist/mnist.cc:74,80; examples/ptb/ptb_rnnlm_lstm.cc:
+ * 101-109), and the optimizers scale and subtract (primitiv/core/
+ * optimizer_impl.cc:22-24).  These entry points stand behind the
+ * corresponding Device virtuals (primitiv/core/device.h:393-479,531-534); an
+ * operation code selects the member of a family.  Formulas follow
+ * primitiv/devices/naive/ops/ and primitiv/devices/cuda/ops/ (file per code
+ * named below).  All are streaming kernels: every operand an operation needs
+ * is read once, every result written once; forward results overwrite,
+ * gradients are accumulated into (`+=`), as in the reference.  The 16-bit
+ * variants read and write 16-bit storage and compute in fp32
+ * (primitiv/devices/cuda16/ops/common.h:16-113). */
+
+/* y = f(x); gx += f'(x, y) * gy over n elements.
+ * Reference: CUDADEV_KERNEL_FW_X / _BW_X (primitiv/devices/cuda/ops/common.h:
+ * 14-28) instantiated in negate.cu, abs.cu, sqrt.cu, exp.cu, log.cu, tanh.cu,
+ * sigmoid.cu, softplus.cu, sin.cu, cos.cu, tan.cu; same formulas in
+ * primitiv/devices/naive/ops/.  The reference has no negate_bw, so
+ * PHIP_NEGATE is forward only.  A backward call reads only those of x and y
+ * that its formula uses; the other may be NULL. */
+typedef enum phip_unary_op {
+  PHIP_NEGATE = 0,
+  PHIP_ABS = 1,
+  PHIP_SQRT = 2,
+  PHIP_EXP = 3,
+  PHIP_LOG = 4,
+  PHIP_TANH = 5,
+  PHIP_SIGMOID = 6,
+  PHIP_SOFTPLUS = 7,
+  PHIP_SIN = 8,
+  PHIP_COS = 9,
+  PHIP_TAN = 10
+} phip_unary_op;
+int phip_unary_fw_f32(phip_ctx *ctx, int op, const float *x, float *y, size_t n);
+int phip_unary_fw_f16(phip_ctx *ctx, int op, const void *x, void *y, size_t n);
+int phip_unary_fw_bf16(phip_ctx *ctx, int op, const void *x, void *y, size_t n);
+int phip_unary_bw_f32(phip_ctx *ctx, int op, const float *x, const float *y, const float *gy, float *gx, size_t n);
+int phip_unary_bw_f16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, void *gx, size_t n);
+int phip_unary_bw_bf16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, void *gx, size_t n);
+
+/* y = f(x, k); gx += df/dx(x, y, k) * gy with a host constant k.
+ * Reference: CUDADEV_KERNEL_FW_X_CONST / _BW_X_CONST (common.h:30-45) in
+ * add.cu, subtract.cu, multiply.cu, divide.cu, pow.cu, prelu.cu, elu.cu.
+ * _R: the constant is the right operand (x - k, x / k, x ^ k); _L: the left
+ * (k - x, k / x, k ^ x).  PRELU: max(x,0) + k*min(x,0); ELU: max(x,0) +
+ * k*(exp(min(x,0)) - 1). */
+typedef enum phip_const_op {
+  PHIP_ADD_CONST = 0,
+  PHIP_SUBTRACT_CONST_R = 1,
+  PHIP_SUBTRACT_CONST_L = 2,
+  PHIP_MULTIPLY_CONST = 3,
+  PHIP_DIVIDE_CONST_R = 4,
+  PHIP_DIVIDE_CONST_L = 5,
+  PHIP_POW_CONST_R = 6,
+  PHIP_POW_CONST_L = 7,
+  PHIP_PRELU = 8,
+  PHIP_ELU = 9
+} phip_const_op;
+int phip_const_fw_f32(phip_ctx *ctx, int op, const float *x, float k, float *y, size_t n);
+int phip_const_fw_f16(phip_ctx *ctx, int op, const void *x, float k, void *y, size_t n);
+int phip_const_fw_bf16(phip_ctx *ctx, int op, const void *x, float k, void *y, size_t n);
+int phip_const_bw_f32(phip_ctx *ctx, int op, const float *x, const float *y, const float *gy, float k, float *gx, size_t n);
+int phip_const_bw_f16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, float k, void *gx, size_t n);
+int phip_const_bw_bf16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, float k, void *gx, size_t n);
+
+/* y = x ^ k for an integer k by repeated squaring; gx += k * gy * y / x.
+ * Reference: pown_fw_impl / pown_bw_impl (primitiv/devices/cuda/ops/pown.cu:
+ * 9-60, primitiv/devices/naive/ops/pown.cc:12-46). */
+int phip_pown_fw_f32(phip_ctx *ctx, const float *x, int32_t k, float *y, size_t n);
+int phip_pown_fw_f16(phip_ctx *ctx, const void *x, int32_t k, void *y, size_t n);
+int phip_pown_fw_bf16(phip_ctx *ctx, const void *x, int32_t k, void *y, size_t n);
+int phip_pown_bw_f32(phip_ctx *ctx, const float *x, const float *y, const float *gy, int32_t k, float *gx, size_t n);
+int phip_pown_bw_f16(phip_ctx *ctx, const void *x, const void *y, const void *gy, int32_t k, void *gx, size_t n);
+int phip_pown_bw_bf16(phip_ctx *ctx, const void *x, const void *y, const void *gy, int32_t k, void *gx, size_t n);
+
+/* Binary operations with minibatch broadcasting.  a holds volume*ba elements,
+ * b volume*bb, y volume*max(ba,bb); ba == bb or one of them is 1.
+ * Forward: y = a op b.  Backward: ga += dy/da * gy, gb += dy/db * gy, where the
+ * gradient of an operand whose batch is 1 is summed over the minibatch (the
+ * reference does this with atomicAdd; here one workgroup owns each output
+ * element and adds in a fixed order).  A backward call reads only those of
+ * a, b, y that its formula uses; the others may be NULL.
+ * Reference: CUDADEV_KERNEL_FW_AB (common.h:65-72) and the *_bw_dev kernels in
+ * add.cu:16-27, subtract.cu, multiply.cu, divide.cu, pow.cu; primitiv/devices/naive/ops/{add,subtract,multiply,divide,
+ * pow}.cc. */
+typedef enum phip_binary_op {
+  PHIP_ADD = 0,
+  PHIP_SUBTRACT = 1,
+  PHIP_MULTIPLY = 2,
+  PHIP_DIVIDE = 3,
+  PHIP_POW = 4
+} phip_binary_op;
+int phip_binary_fw_f32(phip_ctx *ctx, int op, const float *a, const float *b, float *y, uint32_t volume, uint32_t ba, uint32_t bb);
+int phip_binary_fw_f16(phip_ctx *ctx, int op, const void *a, const void *b, void *y, uint32_t volume, uint32_t ba, uint32_t bb);
+int phip_binary_fw_bf16(phip_ctx *ctx, int op, const void *a, const void *b, void *y, uint32_t volume, uint32_t ba, uint32_t bb);
+int phip_binary_bw_f32(phip_ctx *ctx, int op, const float *a, const float *b, const float *y, const float *gy,
+                       float *ga, float *gb, uint32_t volume, uint32_t ba, uint32_t bb);
+int phip_binary_bw_f16(phip_ctx *ctx, int op, const void *a, const void *b, const void *y, const void *gy,
+                       void *ga, void *gb, uint32_t volume, uint32_t ba, uint32_t bb);
+int phip_binary_bw_bf16(phip_ctx *ctx, int op, const void *a, const void *b, const void *y, const void *gy,
+                       void *ga, void *gb, uint32_t volume, uint32_t ba, uint32_t bb);
+
+/* y = x op k (k_on_left == 0) or k op x (k_on_left != 0), where k holds one
+ * scalar per sample: x has volume*bx elements, k has bk, y volume*max(bx,bk).
+ * Reference: CUDADEV_KERNEL_FW_X_SCALAR_R / _L (common.h:47-63) for
+ * add_scalar, subtract_scalar_{r,l}, multiply_scalar, divide_scalar_{r,l},
+ * pow_scalar_{r,l}; CPUDEV_FW_X_SCALAR (primitiv/devices/naive/ops/common.h:
+ * 50-68). */
+int phip_scalar_fw_f32(phip_ctx *ctx, int op, int k_on_left, const float *x, const float *k, float *y,
+                       uint32_t volume, uint32_t bx, uint32_t bk);
+int phip_scalar_fw_f16(phip_ctx *ctx, int op, int k_on_left, const void *x, const void *k, void *y,
+                       uint32_t volume, uint32_t bx, uint32_t bk);
+int phip_scalar_fw_bf16(phip_ctx *ctx, int op, int k_on_left, const void *x, const void *k, void *y,
+                       uint32_t volume, uint32_t bx, uint32_t bk);
+
+/* y -= x with minibatch broadcasting (same operand rules as phip_inplace_add).
+ * Reference: inplace_subtract_impl (primitiv/devices/cuda/ops/
+ * inplace_subtract.cu:9-27, primitiv/devices/naive/ops/inplace_subtract.cc:
+ * 11-27). */
+int phip_inplace_subtract_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bx, uint32_t by);
+int phip_inplace_subtract_f16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by);
+int phip_inplace_subtract_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by);
+
+/* x *= k over n elements.
+ * Reference: inplace_multiply_const_impl (primitiv/devices/cuda/ops/
+ * inplace_multiply_const.cu:9-23). */
+int phip_inplace_multiply_const_f32(phip_ctx *ctx, float k, float *x, size_t n);
+int phip_inplace_multiply_const_f16(phip_ctx *ctx, float k, void *x, size_t n);
+int phip_inplace_multiply_const_bf16(phip_ctx *ctx, float k, void *x, size_t n);
+
+/* y = identity matrix of `rows` x `rows`.
+ * Reference: identity_impl (primitiv/devices/cuda/ops/identity.cu:9-22). */
+int phip_identity_f32(phip_ctx *ctx, float *y, uint32_t rows);
+int phip_identity_f16(phip_ctx *ctx, void *y, uint32_t rows);
+int phip_identity_bf16(phip_ctx *ctx, void *y, uint32_t rows);
+
 /* ---- timing ---------------------------------------------------------------
  * No counterpart in the reference (it has no profiling facility); events are
  * recorded on the context's stream so they bracket exactly the kernels the

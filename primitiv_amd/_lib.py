@@ -82,6 +82,42 @@ SIGNATURES = {
     "phip_batch_sum_f32": [_vp, _vp, _vp, _u32, _u32],
     "phip_batch_sum_f16": [_vp, _vp, _vp, _u32, _u32],
     "phip_batch_sum_bf16": [_vp, _vp, _vp, _u32, _u32],
+    "phip_unary_fw_f32": [_vp, _int, _vp, _vp, _sz],
+    "phip_unary_bw_f32": [_vp, _int, _vp, _vp, _vp, _vp, _sz],
+    "phip_const_fw_f32": [_vp, _int, _vp, _f, _vp, _sz],
+    "phip_const_bw_f32": [_vp, _int, _vp, _vp, _vp, _f, _vp, _sz],
+    "phip_pown_fw_f32": [_vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_pown_bw_f32": [_vp, _vp, _vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_binary_fw_f32": [_vp, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_binary_bw_f32": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_scalar_fw_f32": [_vp, _int, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_subtract_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_multiply_const_f32": [_vp, _f, _vp, _sz],
+    "phip_identity_f32": [_vp, _vp, _u32],
+    "phip_unary_fw_f16": [_vp, _int, _vp, _vp, _sz],
+    "phip_unary_bw_f16": [_vp, _int, _vp, _vp, _vp, _vp, _sz],
+    "phip_const_fw_f16": [_vp, _int, _vp, _f, _vp, _sz],
+    "phip_const_bw_f16": [_vp, _int, _vp, _vp, _vp, _f, _vp, _sz],
+    "phip_pown_fw_f16": [_vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_pown_bw_f16": [_vp, _vp, _vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_binary_fw_f16": [_vp, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_binary_bw_f16": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_scalar_fw_f16": [_vp, _int, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_subtract_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_multiply_const_f16": [_vp, _f, _vp, _sz],
+    "phip_identity_f16": [_vp, _vp, _u32],
+    "phip_unary_fw_bf16": [_vp, _int, _vp, _vp, _sz],
+    "phip_unary_bw_bf16": [_vp, _int, _vp, _vp, _vp, _vp, _sz],
+    "phip_const_fw_bf16": [_vp, _int, _vp, _f, _vp, _sz],
+    "phip_const_bw_bf16": [_vp, _int, _vp, _vp, _vp, _f, _vp, _sz],
+    "phip_pown_fw_bf16": [_vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_pown_bw_bf16": [_vp, _vp, _vp, _vp, ctypes.c_int32, _vp, _sz],
+    "phip_binary_fw_bf16": [_vp, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_binary_bw_bf16": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_scalar_fw_bf16": [_vp, _int, _int, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_subtract_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_inplace_multiply_const_bf16": [_vp, _f, _vp, _sz],
+    "phip_identity_bf16": [_vp, _vp, _u32],
     "phip_matmul_fw_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_f16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_bf16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],

@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(HERE, "libphip.so")
 SOURCES = [
     "phip_runtime.hip",
     "phip_elementwise.hip",
+    "phip_pointwise_unary.hip",
+    "phip_pointwise_binary.hip",
     "phip_gemm_f32.hip",
     "phip_gemm_f32_direct.hip",
     "phip_gemm_f32_lds.hip",

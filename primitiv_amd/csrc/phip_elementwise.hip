@@ -1,5 +1,5 @@
 // Streaming helpers around the matmul path: fill, storage conversion,
-// broadcasting in-place add and minibatch sum.  All are HBM-bound; each
+// broadcasting in-place add / subtract and minibatch sum.  All are HBM-bound; each
 // element is read once and written once.
 #include "phip_internal.h"
 #include "phip_types.h"
@@ -29,26 +29,26 @@ __global__ __launch_bounds__(kBlock) void cvt_kernel(const S *__restrict__ src, 
   }
 }
 
-// y[n][i] += x[n or 0][i]   (by == bs; x advances only when it has a batch)
+// y[n][i] += sign * x[n or 0][i]   (by == bs; x advances only when it has a batch)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void add_same_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                          size_t volume, size_t total, bool x_batched) {
+                                                          size_t volume, size_t total, bool x_batched, float sign) {
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (size_t)gridDim.x * kBlock) {
     const size_t xi = x_batched ? i : i % volume;
-    y[i] = from_f32<T>(to_f32(y[i]) + to_f32(x[xi]));
+    y[i] = from_f32<T>(to_f32(y[i]) + sign * to_f32(x[xi]));
   }
 }
 
-// y[i] (+)= sum_n x[n][i]; one thread owns one output element, so the
+// y[i] (+)= sign * sum_n x[n][i]; one thread owns one output element, so the
 // reduction needs no atomics and its order is fixed.
 template <typename T, bool kAccumulate>
 __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                              size_t volume, uint32_t bs) {
+                                                              size_t volume, uint32_t bs, float sign) {
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < volume; i += (size_t)gridDim.x * kBlock) {
     float s = kAccumulate ? to_f32(y[i]) : 0.0f;
     const T *px = x + i;
     for (uint32_t n = 0; n < bs; ++n) {
-      s += to_f32(*px);
+      s += sign * to_f32(*px);
       px += volume;
     }
     y[i] = from_f32<T>(s);
@@ -79,7 +79,7 @@ static int cvt_impl(phip_ctx *ctx, const void *src, void *dst, size_t n) {
 
 template <typename T>
 static int inplace_add_impl(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx,
-                            uint32_t by) {
+                            uint32_t by, float sign) {
   PHIP_ENTER(ctx);
   PHIP_REQUIRE(bx >= 1 && by >= 1 && (bx == by || bx == 1 || by == 1),
                "incompatible batch sizes: %u, %u", bx, by);
@@ -87,11 +87,11 @@ static int inplace_add_impl(phip_ctx *ctx, const void *x, void *y, uint32_t volu
   PHIP_REQUIRE(x != nullptr && y != nullptr, "null pointer");
   if (by == 1 && bx > 1) {
     hipLaunchKernelGGL((batch_reduce_kernel<T, true>), dim3(grid_for(volume, 1, ctx)), dim3(kBlock), 0,
-                       ctx->stream, static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, bx);
+                       ctx->stream, static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, bx, sign);
   } else {
     const size_t total = (size_t)volume * by;
     hipLaunchKernelGGL(add_same_kernel<T>, dim3(grid_for(total, 4, ctx)), dim3(kBlock), 0, ctx->stream,
-                       static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, total, bx > 1);
+                       static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, total, bx > 1, sign);
   }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
@@ -104,7 +104,7 @@ static int batch_sum_impl(phip_ctx *ctx, const void *x, void *y, uint32_t volume
   if (volume == 0) return PHIP_OK;
   PHIP_REQUIRE(x != nullptr && y != nullptr, "null pointer");
   hipLaunchKernelGGL((batch_reduce_kernel<T, false>), dim3(grid_for(volume, 1, ctx)), dim3(kBlock), 0,
-                     ctx->stream, static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, bs);
+                     ctx->stream, static_cast<const T *>(x), static_cast<T *>(y), (size_t)volume, bs, 1.0f);
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
 }
@@ -125,13 +125,23 @@ int phip_cvt_f32_to_bf16(phip_ctx *ctx, const float *s, void *d, size_t n) { ret
 int phip_cvt_bf16_to_f32(phip_ctx *ctx, const void *s, float *d, size_t n) { return cvt_impl<bf16_t, float>(ctx, s, d, n); }
 
 int phip_inplace_add_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bx, uint32_t by) {
-  return inplace_add_impl<float>(ctx, x, y, volume, bx, by);
+  return inplace_add_impl<float>(ctx, x, y, volume, bx, by, 1.0f);
 }
 int phip_inplace_add_f16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by) {
-  return inplace_add_impl<f16_t>(ctx, x, y, volume, bx, by);
+  return inplace_add_impl<f16_t>(ctx, x, y, volume, bx, by, 1.0f);
 }
 int phip_inplace_add_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by) {
-  return inplace_add_impl<bf16_t>(ctx, x, y, volume, bx, by);
+  return inplace_add_impl<bf16_t>(ctx, x, y, volume, bx, by, 1.0f);
+}
+
+int phip_inplace_subtract_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bx, uint32_t by) {
+  return inplace_add_impl<float>(ctx, x, y, volume, bx, by, -1.0f);
+}
+int phip_inplace_subtract_f16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by) {
+  return inplace_add_impl<f16_t>(ctx, x, y, volume, bx, by, -1.0f);
+}
+int phip_inplace_subtract_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t volume, uint32_t bx, uint32_t by) {
+  return inplace_add_impl<bf16_t>(ctx, x, y, volume, bx, by, -1.0f);
 }
 
 int phip_batch_sum_f32(phip_ctx *ctx, const float *x, float *y, uint32_t volume, uint32_t bs) {

@@ -107,6 +107,22 @@ class shape_ops:
     def batch_sum(x):
         return x.resize_batch(1)
 
+    @staticmethod
+    def elementwise(a, b):
+        # shape_ops.cc:34-41
+        if not a.has_same_dims(b) or not a.has_compatible_batch(b):
+            raise Error("Shape mismatched for the elementwise operation. a: %s != b: %s"
+                        % (a.to_string(), b.to_string()))
+        return a.resize_batch(max(a.batch(), b.batch()))
+
+    @staticmethod
+    def scalar_op(x, k):
+        # shape_ops.cc:25-32
+        if k.volume() != 1 or k.depth() != 0 or not x.has_compatible_batch(k):
+            raise Error("Shape mismatched for the scalar operation. x: %s != k: %s"
+                        % (x.to_string(), k.to_string()))
+        return x.resize_batch(max(x.batch(), k.batch()))
+
 
 class _Handle:
     """One pool block; returned to the pool of its context when dropped,
@@ -382,6 +398,128 @@ class HIP:
         y = self.new_raw_tensor(shape_ops.batch_sum(x.shape()))
         _lib.call("phip_batch_sum_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(),
                   x.shape().volume(), x.shape().batch())
+        return y
+
+    # -- elementwise operations around the matmul ------------------------------
+    # Operation codes of include/phip.h.
+    UNARY_OPS = ("negate", "abs", "sqrt", "exp", "log", "tanh", "sigmoid", "softplus", "sin", "cos", "tan")
+    CONST_OPS = ("add_const", "subtract_const_r", "subtract_const_l", "multiply_const", "divide_const_r",
+                 "divide_const_l", "pow_const_r", "pow_const_l", "prelu", "elu")
+    BINARY_OPS = ("add", "subtract", "multiply", "divide", "pow")
+    # scalar operation -> (binary operation, scalar on the left)
+    SCALAR_OPS = {"add_scalar": ("add", False), "subtract_scalar_r": ("subtract", False),
+                  "subtract_scalar_l": ("subtract", True), "multiply_scalar": ("multiply", False),
+                  "divide_scalar_r": ("divide", False), "divide_scalar_l": ("divide", True),
+                  "pow_scalar_r": ("pow", False), "pow_scalar_l": ("pow", True)}
+
+    def _bw_x_check(self, name, x, y, gy, gx):
+        # DEV_BW_X / DEV_BW_X_CONST, device.cc:221-266
+        for t in (x, y, gy, gx):
+            self._check_device(t)
+        s = x.shape()
+        if y.shape() != s or gy.shape() != s or gx.shape() != s:
+            raise Error("Shape mismatched at %s_bw. x.shape: %s, y.shape: %s, gy.shape: %s, gx.shape: %s"
+                        % ((name,) + tuple(t.shape().to_string() for t in (x, y, gy, gx))))
+
+    def unary_fw(self, op, x):
+        """`op`_fw(x) for an op of UNARY_OPS (DEV_FW_X, device.cc:213-219,303-313)."""
+        self._check_device(x)
+        y = self.new_raw_tensor(x.shape())
+        _lib.call("phip_unary_fw_" + self._SUFFIX, self._ctx, self.UNARY_OPS.index(op), x.handle(),
+                  y.mutable_handle(), x.shape().size())
+        return y
+
+    def unary_bw(self, op, x, y, gy, gx):
+        self._bw_x_check(op, x, y, gy, gx)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_unary_bw_" + self._SUFFIX, self._ctx, self.UNARY_OPS.index(op), x.handle(), y.handle(),
+                  gy.handle(), pgx, x.shape().size())
+
+    def const_fw(self, op, x, k):
+        """`op`_fw(x, k) for an op of CONST_OPS (DEV_FW_X_CONST, device.cc:241-247)."""
+        self._check_device(x)
+        y = self.new_raw_tensor(x.shape())
+        _lib.call("phip_const_fw_" + self._SUFFIX, self._ctx, self.CONST_OPS.index(op), x.handle(), float(k),
+                  y.mutable_handle(), x.shape().size())
+        return y
+
+    def const_bw(self, op, x, y, gy, k, gx):
+        self._bw_x_check(op, x, y, gy, gx)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_const_bw_" + self._SUFFIX, self._ctx, self.CONST_OPS.index(op), x.handle(), y.handle(),
+                  gy.handle(), float(k), pgx, x.shape().size())
+
+    def pown_fw(self, x, k):
+        self._check_device(x)
+        y = self.new_raw_tensor(x.shape())
+        _lib.call("phip_pown_fw_" + self._SUFFIX, self._ctx, x.handle(), int(k), y.mutable_handle(),
+                  x.shape().size())
+        return y
+
+    def pown_bw(self, x, y, gy, k, gx):
+        self._bw_x_check("pown", x, y, gy, gx)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_pown_bw_" + self._SUFFIX, self._ctx, x.handle(), y.handle(), gy.handle(), int(k), pgx,
+                  x.shape().size())
+
+    def scalar_fw(self, op, x, k):
+        """`op`_fw(x, k) for an op of SCALAR_OPS; k holds one scalar per sample
+        (DEV_FW_AB with shape_ops::scalar_op, device.cc:404-411)."""
+        self._check_device(x)
+        self._check_device(k)
+        y = self.new_raw_tensor(shape_ops.scalar_op(x.shape(), k.shape()))
+        binary, left = self.SCALAR_OPS[op]
+        _lib.call("phip_scalar_fw_" + self._SUFFIX, self._ctx, self.BINARY_OPS.index(binary), int(left),
+                  x.handle(), k.handle(), y.mutable_handle(), x.shape().volume(), x.shape().batch(),
+                  k.shape().batch())
+        return y
+
+    def binary_fw(self, op, a, b):
+        """`op`_fw(a, b) for an op of BINARY_OPS (DEV_FW_AB, device.cc:268-275,413-417)."""
+        self._check_device(a)
+        self._check_device(b)
+        y = self.new_raw_tensor(shape_ops.elementwise(a.shape(), b.shape()))
+        _lib.call("phip_binary_fw_" + self._SUFFIX, self._ctx, self.BINARY_OPS.index(op), a.handle(), b.handle(),
+                  y.mutable_handle(), y.shape().volume(), a.shape().batch(), b.shape().batch())
+        return y
+
+    def binary_bw(self, op, a, b, y, gy, ga, gb):
+        # DEV_BW_AB, device.cc:277-301,448-452
+        for t in (a, b, y, gy, ga, gb):
+            self._check_device(t)
+        if (a.shape() != ga.shape() or b.shape() != gb.shape() or y.shape() != gy.shape()
+                or y.shape() != shape_ops.elementwise(a.shape(), b.shape())):
+            raise Error("Shape mismatched at %s_bw. a: %s, b: %s, y: %s, gy: %s, ga: %s, gb: %s"
+                        % ((op,) + tuple(t.shape().to_string() for t in (a, b, y, gy, ga, gb))))
+        pga, pgb = ga.mutable_handle(), gb.mutable_handle()
+        _lib.call("phip_binary_bw_" + self._SUFFIX, self._ctx, self.BINARY_OPS.index(op), a.handle(), b.handle(),
+                  y.handle(), gy.handle(), pga, pgb, y.shape().volume(), a.shape().batch(), b.shape().batch())
+
+    def inplace_multiply_const(self, k, x):
+        # device.cc:687-690
+        self._check_device(x)
+        _lib.call("phip_inplace_multiply_const_" + self._SUFFIX, self._ctx, float(k), x.mutable_handle(),
+                  x.shape().size())
+        return x
+
+    def inplace_subtract(self, x, y):
+        # device.cc:705-716
+        self._check_device(x)
+        self._check_device(y)
+        sx, sy = x.shape(), y.shape()
+        if not sx.has_same_dims(sy) or not sx.has_compatible_batch(sy):
+            raise Error("Attempted to subtract values of shape %s from shape %s"
+                        % (sx.to_string(), sy.to_string()))
+        _lib.call("phip_inplace_subtract_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(),
+                  sy.volume(), sx.batch(), sy.batch())
+        return y
+
+    def identity(self, size):
+        # device.cc:98-105
+        if size == 0:
+            raise Error("Invalid size of the identity matrix. size: 0")
+        y = self.new_raw_tensor(Shape([size, size]))
+        _lib.call("phip_identity_" + self._SUFFIX, self._ctx, y.mutable_handle(), size)
         return y
 
 

@@ -30,6 +30,8 @@ find_program(PRIMITIV_HIPCC hipcc HINTS "${ROCM_PATH}/bin" REQUIRED)
 set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_runtime.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_elementwise.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_pointwise_unary.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_pointwise_binary.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_direct.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip
