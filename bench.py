@@ -147,6 +147,78 @@ def measure(name, steps, warmup, skip_cpu):
     return out
 
 
+def _event_seconds(dev, fn, reps):
+    """Average seconds of one fn() over `reps` back-to-back calls, by events on the library's stream."""
+    ctx = dev.ctx()
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    _lib.call("phip_event_create", ctx, ctypes.byref(e0))
+    _lib.call("phip_event_create", ctx, ctypes.byref(e1))
+    for _ in range(2):
+        fn()
+    dev.sync()
+    _lib.call("phip_event_record", ctx, e0)
+    for _ in range(reps):
+        fn()
+    _lib.call("phip_event_record", ctx, e1)
+    ms = ctypes.c_float()
+    _lib.call("phip_event_elapsed_ms", e0, e1, ctypes.byref(ms))
+    _lib.call("phip_event_destroy", e0)
+    _lib.call("phip_event_destroy", e1)
+    return ms.value * 1e-3 / reps
+
+
+def measure_pointwise(reps=20):
+    """Streaming rate of the elementwise kernels: algorithmic bytes (every operand the
+    operation needs read once, every result written once, a gradient read and written)
+    over the event time, against the 8 TB/s HBM peak.  Large cases are 64 Mi elements per
+    tensor; the bias cases use a 1 Mi-element bias over a minibatch of 64, and the
+    recurrent-layer shape (2048 x 64) shows the latency floor."""
+    S = pa.Shape
+    out = []
+    for storage, item in (("f32", 4), ("f16", 2)):
+        dev = pa.HIP(0) if storage == "f32" else pa.HIP16(0, storage=storage)
+        n = 64 << 20
+        x = dev.new_tensor_by_constant(S([n]), 0.5)
+        y = dev.new_tensor_by_constant(S([n]), 0.25)
+        g = dev.new_tensor_by_constant(S([n]), 0.0)
+        g2 = dev.new_tensor_by_constant(S([n]), 0.0)
+        vol, bs = 1 << 20, 64
+        bias = dev.new_tensor_by_constant(S([vol]), 0.5)
+        gbias = dev.new_tensor_by_constant(S([vol]), 0.0)
+        xb = dev.new_tensor_by_constant(S([vol], bs), 0.5)
+        gxb = dev.new_tensor_by_constant(S([vol], bs), 0.0)
+        sv, sb = 2048, 64
+        sbias = dev.new_tensor_by_constant(S([sv]), 0.5)
+        sx = dev.new_tensor_by_constant(S([sv], sb), 0.5)
+        sg = dev.new_tensor_by_constant(S([sv], sb), 0.0)
+        sgb = dev.new_tensor_by_constant(S([sv]), 0.0)
+        big, med = n * item, vol * bs * item
+        cases = [
+            ("tanh_fw", lambda: dev.unary_fw("tanh", x), 2 * big),
+            ("tanh_bw", lambda: dev.unary_bw("tanh", x, y, x, g), 4 * big),
+            ("prelu_fw", lambda: dev.const_fw("prelu", x, 0.01), 2 * big),
+            ("add_fw", lambda: dev.binary_fw("add", x, y), 3 * big),
+            ("multiply_bw", lambda: dev.binary_bw("multiply", x, y, x, y, g, g2), 7 * big),
+            ("bias_add_fw", lambda: dev.binary_fw("add", xb, bias), 2 * med + vol * item),
+            ("bias_add_bw", lambda: dev.binary_bw("add", xb, bias, xb, xb, gxb, gbias), 3 * med + 2 * vol * item),
+            ("inplace_add", lambda: dev.inplace_add(x, y), 3 * big),
+            ("inplace_multiply_const", lambda: dev.inplace_multiply_const(1.0, y), 2 * big),
+            ("bias_add_fw_2048x64", lambda: dev.binary_fw("add", sx, sbias), (2 * sv * sb + sv) * item),
+            ("bias_add_bw_2048x64", lambda: dev.binary_bw("add", sx, sbias, sx, sx, sg, sgb),
+             (3 * sv * sb + 2 * sv) * item),
+        ]
+        for name, fn, nbytes in cases:
+            sec = _event_seconds(dev, fn, reps)
+            out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
+                        "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
+            print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
+                  % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
+                  file=sys.stderr, flush=True)
+        del x, y, g, g2, bias, gbias, xb, gxb, sbias, sx, sg, sgb, cases
+        dev.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -157,10 +229,16 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one streaming y += x over 64 Mi floats (reads 512 MiB, writes 256 MiB): "
                          "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--pointwise", action="store_true",
+                    help="measure the elementwise kernels' streaming rates instead of the matmul workloads")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path "
                  "(run with --gpus 1).")
+    if args.pointwise:
+        print(json.dumps({"metric": "elementwise kernels, algorithmic GB/s", "unit": "GB/s", "n_gpus": 1,
+                          "peak": PEAK_HBM_GBS, "data": "synthetic", "kernels": measure_pointwise()}))
+        return
 
     if args.traffic_calibration:
         dev = pa.HIP(0)

@@ -30,6 +30,71 @@ const char *suffix_name(primitiv::devices::HIP::Storage s) {
   }
 }
 
+// libphip's elementwise entry points for one storage type, behind one
+// signature (the fp32 variants take float pointers, the 16-bit ones void).
+struct PointwiseAbi {
+  int (*unary_fw)(phip_ctx *, int, const void *, void *, size_t);
+  int (*unary_bw)(phip_ctx *, int, const void *, const void *, const void *, void *, size_t);
+  int (*const_fw)(phip_ctx *, int, const void *, float, void *, size_t);
+  int (*const_bw)(phip_ctx *, int, const void *, const void *, const void *, float, void *, size_t);
+  int (*pown_fw)(phip_ctx *, const void *, std::int32_t, void *, size_t);
+  int (*pown_bw)(phip_ctx *, const void *, const void *, const void *, std::int32_t, void *, size_t);
+  int (*binary_fw)(phip_ctx *, int, const void *, const void *, void *, std::uint32_t, std::uint32_t, std::uint32_t);
+  int (*binary_bw)(phip_ctx *, int, const void *, const void *, const void *, const void *, void *, void *,
+                   std::uint32_t, std::uint32_t, std::uint32_t);
+  int (*scalar_fw)(phip_ctx *, int, int, const void *, const void *, void *, std::uint32_t, std::uint32_t,
+                   std::uint32_t);
+  int (*inplace_subtract)(phip_ctx *, const void *, void *, std::uint32_t, std::uint32_t, std::uint32_t);
+  int (*inplace_multiply_const)(phip_ctx *, float, void *, size_t);
+  int (*identity)(phip_ctx *, void *, std::uint32_t);
+};
+
+typedef const float *CF;
+typedef float *MF;
+
+const PointwiseAbi &pointwise_abi(primitiv::devices::HIP::Storage s) {
+  static const PointwiseAbi f32 = {
+    [](phip_ctx *c, int op, const void *x, void *y, size_t n) {
+      return ::phip_unary_fw_f32(c, op, CF(x), MF(y), n); },
+    [](phip_ctx *c, int op, const void *x, const void *y, const void *gy, void *gx, size_t n) {
+      return ::phip_unary_bw_f32(c, op, CF(x), CF(y), CF(gy), MF(gx), n); },
+    [](phip_ctx *c, int op, const void *x, float k, void *y, size_t n) {
+      return ::phip_const_fw_f32(c, op, CF(x), k, MF(y), n); },
+    [](phip_ctx *c, int op, const void *x, const void *y, const void *gy, float k, void *gx, size_t n) {
+      return ::phip_const_bw_f32(c, op, CF(x), CF(y), CF(gy), k, MF(gx), n); },
+    [](phip_ctx *c, const void *x, std::int32_t k, void *y, size_t n) {
+      return ::phip_pown_fw_f32(c, CF(x), k, MF(y), n); },
+    [](phip_ctx *c, const void *x, const void *y, const void *gy, std::int32_t k, void *gx, size_t n) {
+      return ::phip_pown_bw_f32(c, CF(x), CF(y), CF(gy), k, MF(gx), n); },
+    [](phip_ctx *c, int op, const void *a, const void *b, void *y, std::uint32_t v, std::uint32_t ba,
+       std::uint32_t bb) { return ::phip_binary_fw_f32(c, op, CF(a), CF(b), MF(y), v, ba, bb); },
+    [](phip_ctx *c, int op, const void *a, const void *b, const void *y, const void *gy, void *ga, void *gb,
+       std::uint32_t v, std::uint32_t ba, std::uint32_t bb) {
+      return ::phip_binary_bw_f32(c, op, CF(a), CF(b), CF(y), CF(gy), MF(ga), MF(gb), v, ba, bb); },
+    [](phip_ctx *c, int op, int left, const void *x, const void *k, void *y, std::uint32_t v, std::uint32_t bx,
+       std::uint32_t bk) { return ::phip_scalar_fw_f32(c, op, left, CF(x), CF(k), MF(y), v, bx, bk); },
+    [](phip_ctx *c, const void *x, void *y, std::uint32_t v, std::uint32_t bx, std::uint32_t by) {
+      return ::phip_inplace_subtract_f32(c, CF(x), MF(y), v, bx, by); },
+    [](phip_ctx *c, float k, void *x, size_t n) { return ::phip_inplace_multiply_const_f32(c, k, MF(x), n); },
+    [](phip_ctx *c, void *y, std::uint32_t rows) { return ::phip_identity_f32(c, MF(y), rows); },
+  };
+  static const PointwiseAbi f16 = {
+    ::phip_unary_fw_f16, ::phip_unary_bw_f16, ::phip_const_fw_f16, ::phip_const_bw_f16, ::phip_pown_fw_f16,
+    ::phip_pown_bw_f16, ::phip_binary_fw_f16, ::phip_binary_bw_f16, ::phip_scalar_fw_f16,
+    ::phip_inplace_subtract_f16, ::phip_inplace_multiply_const_f16, ::phip_identity_f16,
+  };
+  static const PointwiseAbi bf16 = {
+    ::phip_unary_fw_bf16, ::phip_unary_bw_bf16, ::phip_const_fw_bf16, ::phip_const_bw_bf16, ::phip_pown_fw_bf16,
+    ::phip_pown_bw_bf16, ::phip_binary_fw_bf16, ::phip_binary_bw_bf16, ::phip_scalar_fw_bf16,
+    ::phip_inplace_subtract_bf16, ::phip_inplace_multiply_const_bf16, ::phip_identity_bf16,
+  };
+  switch (s) {
+    case primitiv::devices::HIP::Storage::F16: return f16;
+    case primitiv::devices::HIP::Storage::BF16: return bf16;
+    default: return f32;
+  }
+}
+
 }  // namespace
 
 namespace primitiv {
@@ -177,11 +242,7 @@ void HIP::copy_tensor_impl(const Tensor &x, Tensor &y) {
 }
 
 void HIP::identity_impl(Tensor &y) {
-  // size x size identity assembled on the host; only used to build constants
-  const std::uint32_t size = y.shape()[0];
-  std::vector<float> host(static_cast<std::size_t>(size) * size, 0.0f);
-  for (std::uint32_t i = 0; i < size; ++i) host[static_cast<std::size_t>(i) * (size + 1)] = 1.0f;
-  reset_tensor_by_array_impl(host.data(), y);
+  PHIP_CALL(pointwise_abi(storage_).identity(ctx_, get_mutable_handle(y), y.shape()[0]));
 }
 
 void HIP::matmul_fw_impl(const Tensor &a, const Tensor &b, Tensor &y) {
@@ -256,6 +317,126 @@ void HIP::inplace_add_impl(const Tensor &x, Tensor &y) {
     case Storage::BF16: PHIP_CALL(::phip_inplace_add_bf16(ctx_, px, py, volume, bx, by)); break;
   }
 }
+
+void HIP::inplace_subtract_impl(const Tensor &x, Tensor &y) {
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(pointwise_abi(storage_).inplace_subtract(
+      ctx_, get_handle(x), py, y.shape().volume(), x.shape().batch(), y.shape().batch()));
+}
+
+void HIP::inplace_multiply_const_impl(float k, Tensor &x) {
+  PHIP_CALL(pointwise_abi(storage_).inplace_multiply_const(ctx_, k, get_mutable_handle(x), x.shape().size()));
+}
+
+// ---- elementwise families ------------------------------------------------------
+// One definition per Device virtual; the libphip operation code names the
+// member (the reference instantiates one kernel per member through
+// CUDADEV_FW_X, CUDADEV_BW_X, ... in primitiv/devices/cuda/ops/common.h:77-151).
+// Writable handles are taken first: taking one may clone a shared block.
+
+void HIP::negate_fw_impl(const Tensor &x, Tensor &y) {
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(pointwise_abi(storage_).unary_fw(ctx_, PHIP_NEGATE, get_handle(x), py, x.shape().size()));
+}
+
+#define PHIP_DEF_X(name, code) \
+void HIP::name##_fw_impl(const Tensor &x, Tensor &y) { \
+  void *py = get_mutable_handle(y); \
+  PHIP_CALL(pointwise_abi(storage_).unary_fw(ctx_, code, get_handle(x), py, x.shape().size())); \
+} \
+void HIP::name##_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, Tensor &gx) { \
+  void *pgx = get_mutable_handle(gx); \
+  PHIP_CALL(pointwise_abi(storage_).unary_bw( \
+      ctx_, code, get_handle(x), get_handle(y), get_handle(gy), pgx, x.shape().size())); \
+}
+
+#define PHIP_DEF_CONST(name, code) \
+void HIP::name##_fw_impl(const Tensor &x, float k, Tensor &y) { \
+  void *py = get_mutable_handle(y); \
+  PHIP_CALL(pointwise_abi(storage_).const_fw(ctx_, code, get_handle(x), k, py, x.shape().size())); \
+} \
+void HIP::name##_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, float k, Tensor &gx) { \
+  void *pgx = get_mutable_handle(gx); \
+  PHIP_CALL(pointwise_abi(storage_).const_bw( \
+      ctx_, code, get_handle(x), get_handle(y), get_handle(gy), k, pgx, x.shape().size())); \
+}
+
+#define PHIP_DEF_SCALAR(name, code, left) \
+void HIP::name##_fw_impl(const Tensor &x, const Tensor &k, Tensor &y) { \
+  void *py = get_mutable_handle(y); \
+  PHIP_CALL(pointwise_abi(storage_).scalar_fw( \
+      ctx_, code, left, get_handle(x), get_handle(k), py, y.shape().volume(), \
+      x.shape().batch(), k.shape().batch())); \
+}
+
+#define PHIP_DEF_AB(name, code) \
+void HIP::name##_fw_impl(const Tensor &a, const Tensor &b, Tensor &y) { \
+  void *py = get_mutable_handle(y); \
+  PHIP_CALL(pointwise_abi(storage_).binary_fw( \
+      ctx_, code, get_handle(a), get_handle(b), py, y.shape().volume(), \
+      a.shape().batch(), b.shape().batch())); \
+} \
+void HIP::name##_bw_impl( \
+    const Tensor &a, const Tensor &b, const Tensor &y, const Tensor &gy, Tensor &ga, Tensor &gb) { \
+  void *pga = get_mutable_handle(ga); \
+  void *pgb = get_mutable_handle(gb); \
+  PHIP_CALL(pointwise_abi(storage_).binary_bw( \
+      ctx_, code, get_handle(a), get_handle(b), get_handle(y), get_handle(gy), pga, pgb, \
+      y.shape().volume(), a.shape().batch(), b.shape().batch())); \
+}
+
+PHIP_DEF_X(abs, PHIP_ABS)
+PHIP_DEF_X(sqrt, PHIP_SQRT)
+PHIP_DEF_X(exp, PHIP_EXP)
+PHIP_DEF_X(log, PHIP_LOG)
+PHIP_DEF_X(tanh, PHIP_TANH)
+PHIP_DEF_X(sigmoid, PHIP_SIGMOID)
+PHIP_DEF_X(softplus, PHIP_SOFTPLUS)
+PHIP_DEF_X(sin, PHIP_SIN)
+PHIP_DEF_X(cos, PHIP_COS)
+PHIP_DEF_X(tan, PHIP_TAN)
+
+PHIP_DEF_CONST(add_const, PHIP_ADD_CONST)
+PHIP_DEF_CONST(subtract_const_r, PHIP_SUBTRACT_CONST_R)
+PHIP_DEF_CONST(subtract_const_l, PHIP_SUBTRACT_CONST_L)
+PHIP_DEF_CONST(multiply_const, PHIP_MULTIPLY_CONST)
+PHIP_DEF_CONST(divide_const_r, PHIP_DIVIDE_CONST_R)
+PHIP_DEF_CONST(divide_const_l, PHIP_DIVIDE_CONST_L)
+PHIP_DEF_CONST(pow_const_r, PHIP_POW_CONST_R)
+PHIP_DEF_CONST(pow_const_l, PHIP_POW_CONST_L)
+PHIP_DEF_CONST(prelu, PHIP_PRELU)
+PHIP_DEF_CONST(elu, PHIP_ELU)
+
+void HIP::pown_fw_impl(const Tensor &x, std::int32_t k, Tensor &y) {
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(pointwise_abi(storage_).pown_fw(ctx_, get_handle(x), k, py, x.shape().size()));
+}
+
+void HIP::pown_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, std::int32_t k, Tensor &gx) {
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(pointwise_abi(storage_).pown_bw(
+      ctx_, get_handle(x), get_handle(y), get_handle(gy), k, pgx, x.shape().size()));
+}
+
+PHIP_DEF_SCALAR(add_scalar, PHIP_ADD, 0)
+PHIP_DEF_SCALAR(subtract_scalar_r, PHIP_SUBTRACT, 0)
+PHIP_DEF_SCALAR(subtract_scalar_l, PHIP_SUBTRACT, 1)
+PHIP_DEF_SCALAR(multiply_scalar, PHIP_MULTIPLY, 0)
+PHIP_DEF_SCALAR(divide_scalar_r, PHIP_DIVIDE, 0)
+PHIP_DEF_SCALAR(divide_scalar_l, PHIP_DIVIDE, 1)
+PHIP_DEF_SCALAR(pow_scalar_r, PHIP_POW, 0)
+PHIP_DEF_SCALAR(pow_scalar_l, PHIP_POW, 1)
+
+PHIP_DEF_AB(add, PHIP_ADD)
+PHIP_DEF_AB(subtract, PHIP_SUBTRACT)
+PHIP_DEF_AB(multiply, PHIP_MULTIPLY)
+PHIP_DEF_AB(divide, PHIP_DIVIDE)
+PHIP_DEF_AB(pow, PHIP_POW)
+
+#undef PHIP_DEF_X
+#undef PHIP_DEF_CONST
+#undef PHIP_DEF_SCALAR
+#undef PHIP_DEF_AB
 
 }  // namespace devices
 }  // namespace primitiv

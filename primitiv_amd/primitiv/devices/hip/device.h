@@ -76,6 +76,38 @@ private:
                       Tensor &ga, Tensor &gb) override;
   void batch_sum_fw_impl(const Tensor &x, Tensor &y) override;
   void inplace_add_impl(const Tensor &x, Tensor &y) override;
+  void inplace_subtract_impl(const Tensor &x, Tensor &y) override;
+  void inplace_multiply_const_impl(float k, Tensor &x) override;
+
+  // elementwise families (libphip operation codes select the member)
+#define PHIP_DECL_X(name) \
+  void name##_fw_impl(const Tensor &x, Tensor &y) override; \
+  void name##_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, Tensor &gx) override;
+#define PHIP_DECL_CONST(name, K) \
+  void name##_fw_impl(const Tensor &x, K k, Tensor &y) override; \
+  void name##_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, K k, Tensor &gx) override;
+#define PHIP_DECL_SCALAR(name) \
+  void name##_fw_impl(const Tensor &x, const Tensor &k, Tensor &y) override;
+#define PHIP_DECL_AB(name) \
+  void name##_fw_impl(const Tensor &a, const Tensor &b, Tensor &y) override; \
+  void name##_bw_impl(const Tensor &a, const Tensor &b, const Tensor &y, const Tensor &gy, \
+                      Tensor &ga, Tensor &gb) override;
+  void negate_fw_impl(const Tensor &x, Tensor &y) override;
+  PHIP_DECL_X(abs) PHIP_DECL_X(sqrt) PHIP_DECL_X(exp) PHIP_DECL_X(log) PHIP_DECL_X(tanh)
+  PHIP_DECL_X(sigmoid) PHIP_DECL_X(softplus) PHIP_DECL_X(sin) PHIP_DECL_X(cos) PHIP_DECL_X(tan)
+  PHIP_DECL_CONST(add_const, float) PHIP_DECL_CONST(subtract_const_r, float)
+  PHIP_DECL_CONST(subtract_const_l, float) PHIP_DECL_CONST(multiply_const, float)
+  PHIP_DECL_CONST(divide_const_r, float) PHIP_DECL_CONST(divide_const_l, float)
+  PHIP_DECL_CONST(pow_const_r, float) PHIP_DECL_CONST(pow_const_l, float) PHIP_DECL_CONST(prelu, float)
+  PHIP_DECL_CONST(elu, float) PHIP_DECL_CONST(pown, std::int32_t)
+  PHIP_DECL_SCALAR(add_scalar) PHIP_DECL_SCALAR(subtract_scalar_r) PHIP_DECL_SCALAR(subtract_scalar_l)
+  PHIP_DECL_SCALAR(multiply_scalar) PHIP_DECL_SCALAR(divide_scalar_r) PHIP_DECL_SCALAR(divide_scalar_l)
+  PHIP_DECL_SCALAR(pow_scalar_r) PHIP_DECL_SCALAR(pow_scalar_l)
+  PHIP_DECL_AB(add) PHIP_DECL_AB(subtract) PHIP_DECL_AB(multiply) PHIP_DECL_AB(divide) PHIP_DECL_AB(pow)
+#undef PHIP_DECL_X
+#undef PHIP_DECL_CONST
+#undef PHIP_DECL_SCALAR
+#undef PHIP_DECL_AB
 
   // ---- not implemented in this backend -------------------------------------
   [[noreturn]] static void unsupported(const char *op);
@@ -84,14 +116,6 @@ private:
   void name##_impl(const Tensor &, Tensor &) override { unsupported(#name); }
 #define PHIP_NI_X_BW(name) \
   void name##_impl(const Tensor &, const Tensor &, const Tensor &, Tensor &) override { unsupported(#name); }
-#define PHIP_NI_CONST(name, K) \
-  void name##_fw_impl(const Tensor &, K, Tensor &) override { unsupported(#name "_fw"); } \
-  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, K, Tensor &) override { unsupported(#name "_bw"); }
-#define PHIP_NI_SCALAR(name) \
-  void name##_fw_impl(const Tensor &, const Tensor &, Tensor &) override { unsupported(#name "_fw"); }
-#define PHIP_NI_AB(name) \
-  void name##_fw_impl(const Tensor &, const Tensor &, Tensor &) override { unsupported(#name "_fw"); } \
-  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, const Tensor &, Tensor &, Tensor &) override { unsupported(#name "_bw"); }
 #define PHIP_NI_DIM(name) \
   void name##_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported(#name "_fw"); }
 #define PHIP_NI_DIM_BW(name) \
@@ -110,28 +134,13 @@ private:
   void pick_bw_impl(const Tensor &, const std::vector<std::uint32_t> &, std::uint32_t, Tensor &) override { unsupported("pick_bw"); }
   void slice_bw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("slice_bw"); }
 
-  PHIP_NI_X(negate_fw) PHIP_NI_X(abs_fw) PHIP_NI_X(sqrt_fw) PHIP_NI_X(exp_fw) PHIP_NI_X(log_fw)
-  PHIP_NI_X(tanh_fw) PHIP_NI_X(sigmoid_fw) PHIP_NI_X(softplus_fw) PHIP_NI_X(sin_fw) PHIP_NI_X(cos_fw)
-  PHIP_NI_X(tan_fw) PHIP_NI_X(transpose_fw)
+  PHIP_NI_X(transpose_fw)
   void permute_dims_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_fw"); }
   void flip_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_fw"); }
 
-  PHIP_NI_X_BW(abs_bw) PHIP_NI_X_BW(sqrt_bw) PHIP_NI_X_BW(exp_bw) PHIP_NI_X_BW(log_bw) PHIP_NI_X_BW(tanh_bw)
-  PHIP_NI_X_BW(sigmoid_bw) PHIP_NI_X_BW(softplus_bw) PHIP_NI_X_BW(sin_bw) PHIP_NI_X_BW(cos_bw)
-  PHIP_NI_X_BW(tan_bw) PHIP_NI_X_BW(transpose_bw)
+  PHIP_NI_X_BW(transpose_bw)
   void permute_dims_bw_impl(const Tensor &, const Tensor &, const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_bw"); }
   void flip_bw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_bw"); }
-
-  PHIP_NI_CONST(add_const, float) PHIP_NI_CONST(subtract_const_r, float) PHIP_NI_CONST(subtract_const_l, float)
-  PHIP_NI_CONST(multiply_const, float) PHIP_NI_CONST(divide_const_r, float) PHIP_NI_CONST(divide_const_l, float)
-  PHIP_NI_CONST(pow_const_r, float) PHIP_NI_CONST(pow_const_l, float) PHIP_NI_CONST(prelu, float)
-  PHIP_NI_CONST(elu, float) PHIP_NI_CONST(pown, std::int32_t)
-
-  PHIP_NI_SCALAR(add_scalar) PHIP_NI_SCALAR(subtract_scalar_r) PHIP_NI_SCALAR(subtract_scalar_l)
-  PHIP_NI_SCALAR(multiply_scalar) PHIP_NI_SCALAR(divide_scalar_r) PHIP_NI_SCALAR(divide_scalar_l)
-  PHIP_NI_SCALAR(pow_scalar_r) PHIP_NI_SCALAR(pow_scalar_l)
-
-  PHIP_NI_AB(add) PHIP_NI_AB(subtract) PHIP_NI_AB(multiply) PHIP_NI_AB(divide) PHIP_NI_AB(pow)
 
   PHIP_NI_DIM(max) PHIP_NI_DIM(min) PHIP_NI_DIM(sum) PHIP_NI_DIM(logsumexp)
   PHIP_NI_DIM_BW(max) PHIP_NI_DIM_BW(min)
@@ -154,14 +163,8 @@ private:
                           std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
                           Tensor &) override { unsupported("max_pool2d_bw"); }
 
-  void inplace_multiply_const_impl(float, Tensor &) override { unsupported("inplace_multiply_const"); }
-  void inplace_subtract_impl(const Tensor &, Tensor &) override { unsupported("inplace_subtract"); }
-
 #undef PHIP_NI_X
 #undef PHIP_NI_X_BW
-#undef PHIP_NI_CONST
-#undef PHIP_NI_SCALAR
-#undef PHIP_NI_AB
 #undef PHIP_NI_DIM
 #undef PHIP_NI_DIM_BW
 #undef PHIP_NI_RANDOM
