@@ -312,6 +312,154 @@ int phip_identity_f32(phip_ctx *ctx, float *y, uint32_t rows);
 int phip_identity_f16(phip_ctx *ctx, void *y, uint32_t rows);
 int phip_identity_bf16(phip_ctx *ctx, void *y, uint32_t rows);
 
+/* ---- moving and reducing along one dimension ---------------------------------
+ * The operations the recurrent and language-model graphs of the reference put
+ * between their matmuls (examples/ptb/ptb_rnnlm_lstm.cc:101-103,146-154;
+ * softmax cross entropy is logsumexp + broadcast + pick, primitiv/core/
+ * tensor_funcs.cc:310-329).  Around a dimension `dim` a tensor is seen as
+ * [outer][n][base]: base = product of the dimensions below dim
+ * (Shape::lower_volume), n = its extent along dim, outer = everything above,
+ * the minibatch included; element (o, j, i) lives at (o*n + j)*base + i. */
+
+/* dst[b][r][i] (= or +=) src[b][r][i] for i < span, r < rows, b < bs, with
+ * element offsets b*bstride + r*stride + i on either side.  A batch stride of
+ * 0 broadcasts the source, or - accumulating only - sums every sample into
+ * the one destination (added in order of b by the thread that owns the
+ * element).  Stands behind slice_fw/bw, concat_fw, batch_slice_fw/bw and
+ * batch_concat_fw, which differ only in the offsets their host side passes
+ * (primitiv/devices/cuda/ops/slice.cu:9-57, concat.cu:9-42, batch_slice.cu:
+ * 9-47, batch_concat.cu:9-32; primitiv/devices/naive/ops/slice.cc:11-56,
+ * concat.cc:11-37). */
+int phip_copy_rows_f32(phip_ctx *ctx, const float *src, float *dst, uint32_t span, uint32_t rows,
+                       uint64_t src_stride, uint64_t dst_stride, uint32_t bs,
+                       uint64_t src_bstride, uint64_t dst_bstride, int accumulate);
+int phip_copy_rows_f16(phip_ctx *ctx, const void *src, void *dst, uint32_t span, uint32_t rows,
+                       uint64_t src_stride, uint64_t dst_stride, uint32_t bs,
+                       uint64_t src_bstride, uint64_t dst_bstride, int accumulate);
+int phip_copy_rows_bf16(phip_ctx *ctx, const void *src, void *dst, uint32_t span, uint32_t rows,
+                       uint64_t src_stride, uint64_t dst_stride, uint32_t bs,
+                       uint64_t src_bstride, uint64_t dst_bstride, int accumulate);
+
+/* pick: y[b][o][0][i] = x[b or 0][o][ids[b or 0]][i]; x is [outer][n][base]
+ * per sample with bx samples, y has bs = max(bx, n_ids) samples; `ids` is a
+ * HOST array of n_ids indices (n_ids == bs, or 1 to use the same index for
+ * every sample), each < n.  Backward: gx[...] += gy, summed over the samples
+ * when bx == 1 (in order of b, no atomics).
+ * Reference: pick_fw_impl / pick_bw_impl (primitiv/devices/cuda/ops/pick.cu:
+ * 9-72, primitiv/devices/naive/ops/pick.cc:11-52). */
+int phip_pick_fw_f32(phip_ctx *ctx, const float *x, const uint32_t *ids, uint32_t n_ids, float *y,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+int phip_pick_fw_f16(phip_ctx *ctx, const void *x, const uint32_t *ids, uint32_t n_ids, void *y,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+int phip_pick_fw_bf16(phip_ctx *ctx, const void *x, const uint32_t *ids, uint32_t n_ids, void *y,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+int phip_pick_bw_f32(phip_ctx *ctx, const float *gy, const uint32_t *ids, uint32_t n_ids, float *gx,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+int phip_pick_bw_f16(phip_ctx *ctx, const void *gy, const uint32_t *ids, uint32_t n_ids, void *gx,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+int phip_pick_bw_bf16(phip_ctx *ctx, const void *gy, const uint32_t *ids, uint32_t n_ids, void *gx,
+                     uint32_t base, uint32_t n, uint32_t outer, uint32_t bx, uint32_t bs);
+
+/* batch_pick: y[b] = x[ids[b]] for whole samples of `volume` elements (x has
+ * bx samples, ids is a HOST array of n_ids indices < bx); backward
+ * gx[ids[b]] += gy[b] in order of b.
+ * Reference: batch_pick_fw_impl / batch_pick_bw_impl (primitiv/devices/cuda/
+ * ops/batch_pick.cu:9-58, primitiv/devices/naive/ops/batch_pick.cc:11-34). */
+int phip_batch_pick_fw_f32(phip_ctx *ctx, const float *x, const uint32_t *ids, uint32_t n_ids, float *y,
+                           uint32_t volume, uint32_t bx);
+int phip_batch_pick_fw_f16(phip_ctx *ctx, const void *x, const uint32_t *ids, uint32_t n_ids, void *y,
+                           uint32_t volume, uint32_t bx);
+int phip_batch_pick_fw_bf16(phip_ctx *ctx, const void *x, const uint32_t *ids, uint32_t n_ids, void *y,
+                           uint32_t volume, uint32_t bx);
+int phip_batch_pick_bw_f32(phip_ctx *ctx, const float *gy, const uint32_t *ids, uint32_t n_ids, float *gx,
+                           uint32_t volume, uint32_t bx);
+int phip_batch_pick_bw_f16(phip_ctx *ctx, const void *gy, const uint32_t *ids, uint32_t n_ids, void *gx,
+                           uint32_t volume, uint32_t bx);
+int phip_batch_pick_bw_bf16(phip_ctx *ctx, const void *gy, const uint32_t *ids, uint32_t n_ids, void *gx,
+                           uint32_t volume, uint32_t bx);
+
+/* Matrix transpose per sample: x is rows x cols, y cols x rows (column-major);
+ * backward gx += transpose(gy) with gx rows x cols.
+ * Reference: transpose_fw_impl / transpose_bw_impl (primitiv/devices/cuda/ops/
+ * transpose.cu:9-54). */
+int phip_transpose_fw_f32(phip_ctx *ctx, const float *x, float *y, uint32_t rows, uint32_t cols, uint32_t bs);
+int phip_transpose_fw_f16(phip_ctx *ctx, const void *x, void *y, uint32_t rows, uint32_t cols, uint32_t bs);
+int phip_transpose_fw_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t rows, uint32_t cols, uint32_t bs);
+int phip_transpose_bw_f32(phip_ctx *ctx, const float *gy, float *gx, uint32_t rows, uint32_t cols, uint32_t bs);
+int phip_transpose_bw_f16(phip_ctx *ctx, const void *gy, void *gx, uint32_t rows, uint32_t cols, uint32_t bs);
+int phip_transpose_bw_bf16(phip_ctx *ctx, const void *gy, void *gx, uint32_t rows, uint32_t cols, uint32_t bs);
+
+/* permute_dims: y's dimension i is x's dimension perm[i]; `dims` are x's
+ * ndims <= 8 extents, `perm` a permutation of 0..ndims-1 (HOST arrays).
+ * Backward: gx += the inverse permutation of gy.
+ * Reference: permute_dims_fw_impl / _bw_impl (primitiv/devices/cuda/ops/
+ * permute_dims.cu:9-115, primitiv/devices/naive/ops/permute_dims.cc:11-84). */
+int phip_permute_dims_fw_f32(phip_ctx *ctx, const float *x, float *y, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+int phip_permute_dims_fw_f16(phip_ctx *ctx, const void *x, void *y, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+int phip_permute_dims_fw_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+int phip_permute_dims_bw_f32(phip_ctx *ctx, const float *gy, float *gx, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+int phip_permute_dims_bw_f16(phip_ctx *ctx, const void *gy, void *gx, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+int phip_permute_dims_bw_bf16(phip_ctx *ctx, const void *gy, void *gx, uint32_t ndims, const uint32_t *dims,
+                             const uint32_t *perm, uint32_t bs);
+
+/* flip: y[o][j][i] = x[o][n-1-j][i]; backward gx[o][j][i] += gy[o][n-1-j][i].
+ * Reference: flip_fw_impl / flip_bw_impl (primitiv/devices/cuda/ops/flip.cu:
+ * 9-63). */
+int phip_flip_fw_f32(phip_ctx *ctx, const float *x, float *y, uint32_t base, uint32_t n, uint32_t outer);
+int phip_flip_fw_f16(phip_ctx *ctx, const void *x, void *y, uint32_t base, uint32_t n, uint32_t outer);
+int phip_flip_fw_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t base, uint32_t n, uint32_t outer);
+int phip_flip_bw_f32(phip_ctx *ctx, const float *gy, float *gx, uint32_t base, uint32_t n, uint32_t outer);
+int phip_flip_bw_f16(phip_ctx *ctx, const void *gy, void *gx, uint32_t base, uint32_t n, uint32_t outer);
+int phip_flip_bw_bf16(phip_ctx *ctx, const void *gy, void *gx, uint32_t base, uint32_t n, uint32_t outer);
+
+/* broadcast: y[o][j][i] = x[o][i] for j < size.
+ * Reference: broadcast_fw_impl (primitiv/devices/cuda/ops/broadcast.cu:9-33). */
+int phip_broadcast_fw_f32(phip_ctx *ctx, const float *x, float *y, uint32_t base, uint32_t size, uint32_t outer);
+int phip_broadcast_fw_f16(phip_ctx *ctx, const void *x, void *y, uint32_t base, uint32_t size, uint32_t outer);
+int phip_broadcast_fw_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t base, uint32_t size, uint32_t outer);
+
+/* Reductions along dim: y[o][i] = op over j < n of x[o][j][i].  The partial
+ * results of the threads that share an output are combined in a fixed order.
+ * Reference: sum_fw_impl, logsumexp_fw_impl, max_fw_impl, min_fw_impl
+ * (primitiv/devices/cuda/ops/sum.cu:9-70, logsumexp.cu:9-80, max.cu:9-43,
+ * 99-123, min.cu; primitiv/devices/naive/ops/{sum,logsumexp,max,min}.cc). */
+typedef enum phip_reduce_op {
+  PHIP_SUM = 0,
+  PHIP_LOGSUMEXP = 1,
+  PHIP_MAX = 2,
+  PHIP_MIN = 3
+} phip_reduce_op;
+int phip_reduce_fw_f32(phip_ctx *ctx, int op, const float *x, float *y, uint32_t base, uint32_t n, uint32_t outer);
+int phip_reduce_fw_f16(phip_ctx *ctx, int op, const void *x, void *y, uint32_t base, uint32_t n, uint32_t outer);
+int phip_reduce_fw_bf16(phip_ctx *ctx, int op, const void *x, void *y, uint32_t base, uint32_t n, uint32_t outer);
+
+/* max_bw / min_bw (op = PHIP_MAX or PHIP_MIN): gx[o][j*][i] += gy[o][i], j*
+ * the first j with x[o][j][i] == y[o][i].
+ * Reference: max_bw_impl / min_bw_impl (primitiv/devices/cuda/ops/max.cu:
+ * 45-97,125-151, primitiv/devices/naive/ops/max.cc:33-55). */
+int phip_extremum_bw_f32(phip_ctx *ctx, int op, const float *x, const float *y, const float *gy, float *gx,
+                         uint32_t base, uint32_t n, uint32_t outer);
+int phip_extremum_bw_f16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, void *gx,
+                         uint32_t base, uint32_t n, uint32_t outer);
+int phip_extremum_bw_bf16(phip_ctx *ctx, int op, const void *x, const void *y, const void *gy, void *gx,
+                         uint32_t base, uint32_t n, uint32_t outer);
+
+/* argmax / argmin (op = PHIP_MAX or PHIP_MIN): host_out[o*base + i] = the
+ * first j attaining the extremum; blocks until the indices are on the host.
+ * Reference: argmax_impl / argmin_impl (primitiv/devices/cuda/ops/argmax.cu:
+ * 9-98, primitiv/devices/naive/ops/argmax.cc:11-36). */
+int phip_arg_extremum_f32(phip_ctx *ctx, int op, const float *x, uint32_t *host_out,
+                          uint32_t base, uint32_t n, uint32_t outer);
+int phip_arg_extremum_f16(phip_ctx *ctx, int op, const void *x, uint32_t *host_out,
+                          uint32_t base, uint32_t n, uint32_t outer);
+int phip_arg_extremum_bf16(phip_ctx *ctx, int op, const void *x, uint32_t *host_out,
+                          uint32_t base, uint32_t n, uint32_t outer);
+
 /* ---- timing ---------------------------------------------------------------
  * No counterpart in the reference (it has no profiling facility); events are
  * recorded on the context's stream so they bracket exactly the kernels the

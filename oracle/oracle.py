@@ -20,6 +20,10 @@ __all__ = [
     "UNARY_OPS", "CONST_OPS", "BINARY_OPS", "unary_fw", "unary_bw", "const_fw",
     "const_bw", "pown_fw", "pown_bw", "scalar_fw", "binary_fw", "binary_bw",
     "inplace_subtract", "inplace_multiply_const", "identity",
+    "REDUCE_OPS", "slice_fw", "slice_bw", "concat_fw", "pick_fw", "pick_bw", "batch_pick_fw",
+    "batch_pick_bw", "batch_slice_fw", "batch_slice_bw", "batch_concat_fw", "transpose_fw",
+    "transpose_bw", "permute_dims_fw", "permute_dims_bw", "flip_fw", "flip_bw", "reduce_fw",
+    "extremum_bw", "arg_extremum", "broadcast_fw",
 ]
 
 _F = ctypes.POINTER(ctypes.c_float)
@@ -77,6 +81,28 @@ def lib():
         l.ref_inplace_multiply_const.restype = None
         l.ref_identity.argtypes = [_F, _U]
         l.ref_identity.restype = None
+        _D = ctypes.POINTER(_U)
+        for name, args in (
+                ("ref_slice_fw", [_F, _D, _U, _U, _U, _U, _U, _F]),
+                ("ref_slice_bw", [_F, _U, _U, _D, _U, _U, _U, _U, _F]),
+                ("ref_concat_fw_one", [_F, _U, _U, _D, _U, _U, _U, _U, _F]),
+                ("ref_pick_fw", [_F, _D, _U, _U, _D, _U, _U, _F]),
+                ("ref_pick_bw", [_F, _D, _U, _U, _D, _U, _U, _F]),
+                ("ref_batch_pick_fw", [_F, _U, _D, _U, _F]),
+                ("ref_batch_pick_bw", [_F, _U, _D, _U, _F]),
+                ("ref_batch_slice_fw", [_F, _U, _U, _U, _F]),
+                ("ref_batch_slice_bw", [_F, _U, _U, _U, _F]),
+                ("ref_transpose_fw", [_F, _U, _U, _U, _F]),
+                ("ref_transpose_bw", [_F, _U, _U, _U, _F]),
+                ("ref_permute_dims_fw", [_F, _D, _U, _D, _U, _F]),
+                ("ref_permute_dims_bw", [_F, _D, _U, _D, _U, _F]),
+                ("ref_flip", [_F, _D, _U, _U, _U, _I, _F]),
+                ("ref_extremum_bw", [_F, _F, _F, _D, _U, _U, _U, _F]),
+                ("ref_arg_extremum", [_I, _F, _D, _U, _U, _U, _D]),
+                ("ref_broadcast_fw", [_F, _D, _U, _U, _U, _U, _F])):
+            getattr(l, name).argtypes = args
+            getattr(l, name).restype = None
+        l.ref_reduce_fw.argtypes = [_I, _F, _D, _U, _U, _U, _F]
         _lib = l
     return _lib
 
@@ -264,4 +290,201 @@ def inplace_multiply_const(k, x):
 def identity(rows):
     y = np.empty(rows * rows, dtype=np.float32)
     lib().ref_identity(_p(y), rows)
+    return y
+
+
+# ---- data movement and reductions (ref_indexing.c) -----------------------------
+# Tensors are (flat float32 array, dims, batch); dims is the list of extents,
+# dimension 0 first, as primitiv's Shape holds them.
+REDUCE_OPS = ["sum", "logsumexp", "max", "min"]
+
+
+def _dims(dims):
+    dims = [int(d) for d in dims]
+    return (_U * max(1, len(dims)))(*dims), len(dims)
+
+
+def _ids(ids):
+    ids = [int(i) for i in ids]
+    return (_U * max(1, len(ids)))(*ids), len(ids)
+
+
+def _vol(dims):
+    v = 1
+    for d in dims:
+        v *= int(d)
+    return v
+
+
+def _dim(dims, i):
+    return int(dims[i]) if i < len(dims) else 1
+
+
+def slice_fw(x, dims, batch, dim, lower, upper):
+    x = _f32(x)
+    assert x.size == _vol(dims) * batch
+    d, depth = _dims(dims)
+    y = np.empty(x.size // _dim(dims, dim) * (upper - lower), dtype=np.float32)
+    lib().ref_slice_fw(_p(x), d, depth, batch, dim, lower, upper - lower, _p(y))
+    return y
+
+
+def slice_bw(gy, by, ny, gx, dims, bx, dim, offset):
+    """Returns gx plus gy placed at `offset` along dim (gx has dims x bx, gy extent ny along dim, batch by)."""
+    gy, gx = _f32(gy), _f32(gx).copy()
+    assert gx.size == _vol(dims) * bx and gy.size == _vol(dims) // _dim(dims, dim) * ny * by
+    d, depth = _dims(dims)
+    lib().ref_slice_bw(_p(gy), by, ny, d, depth, bx, dim, offset, _p(gx))
+    return gx
+
+
+def concat_fw(xs, dim):
+    """xs: list of (array, dims, batch); returns (array, dims, batch) of the concatenation along dim."""
+    dims0 = list(xs[0][1]) + [1] * max(0, dim + 1 - len(xs[0][1]))
+    ydims = list(dims0)
+    ydims[dim] = sum(_dim(x[1], dim) for x in xs)
+    by = max(x[2] for x in xs)
+    y = np.empty(_vol(ydims) * by, dtype=np.float32)
+    d, depth = _dims(ydims)
+    offset = 0
+    for arr, dims, batch in xs:
+        arr = _f32(arr)
+        assert arr.size == _vol(dims) * batch
+        lib().ref_concat_fw_one(_p(arr), _dim(dims, dim), batch, d, depth, by, dim, offset, _p(y))
+        offset += _dim(dims, dim)
+    return y, ydims, by
+
+
+def pick_fw(x, dims, bx, ids, dim):
+    x = _f32(x)
+    assert x.size == _vol(dims) * bx
+    d, depth = _dims(dims)
+    i, n = _ids(ids)
+    y = np.empty(_vol(dims) // _dim(dims, dim) * max(bx, n), dtype=np.float32)
+    lib().ref_pick_fw(_p(x), d, depth, bx, i, n, dim, _p(y))
+    return y
+
+
+def pick_bw(gy, gx, dims, bx, ids, dim):
+    gy, gx = _f32(gy), _f32(gx).copy()
+    d, depth = _dims(dims)
+    i, n = _ids(ids)
+    assert gx.size == _vol(dims) * bx and gy.size == _vol(dims) // _dim(dims, dim) * max(bx, n)
+    lib().ref_pick_bw(_p(gy), d, depth, bx, i, n, dim, _p(gx))
+    return gx
+
+
+def batch_pick_fw(x, volume, ids):
+    x = _f32(x)
+    i, n = _ids(ids)
+    y = np.empty(volume * n, dtype=np.float32)
+    lib().ref_batch_pick_fw(_p(x), volume, i, n, _p(y))
+    return y
+
+
+def batch_pick_bw(gy, gx, volume, ids):
+    gy, gx = _f32(gy), _f32(gx).copy()
+    i, n = _ids(ids)
+    assert gy.size == volume * n
+    lib().ref_batch_pick_bw(_p(gy), volume, i, n, _p(gx))
+    return gx
+
+
+def batch_slice_fw(x, volume, lower, upper):
+    x = _f32(x)
+    y = np.empty(volume * (upper - lower), dtype=np.float32)
+    lib().ref_batch_slice_fw(_p(x), volume, lower, upper - lower, _p(y))
+    return y
+
+
+def batch_slice_bw(gy, gx, volume, offset):
+    gy, gx = _f32(gy), _f32(gx).copy()
+    lib().ref_batch_slice_bw(_p(gy), volume, offset, gy.size // volume, _p(gx))
+    return gx
+
+
+def batch_concat_fw(xs):
+    # naive/ops/batch_concat.cc:11-22: the inputs one after the other
+    return np.concatenate([_f32(x) for x in xs])
+
+
+def transpose_fw(x, d1, d2, bs):
+    x = _f32(x)
+    assert x.size == d1 * d2 * bs
+    y = np.empty_like(x)
+    lib().ref_transpose_fw(_p(x), d1, d2, bs, _p(y))
+    return y
+
+
+def transpose_bw(gy, gx, d1, d2, bs):
+    """gx (d1 x d2 per sample) plus the transpose of gy (d2 x d1)."""
+    gy, gx = _f32(gy), _f32(gx).copy()
+    lib().ref_transpose_bw(_p(gy), d1, d2, bs, _p(gx))
+    return gx
+
+
+def permute_dims_fw(x, dims, perm, bs):
+    x = _f32(x)
+    dims = list(dims) + [1] * (len(perm) - len(dims))
+    d, nd = _dims(dims)
+    pm, _ = _ids(perm)
+    y = np.empty_like(x)
+    lib().ref_permute_dims_fw(_p(x), d, nd, pm, bs, _p(y))
+    return y
+
+
+def permute_dims_bw(gy, gx, dims, perm, bs):
+    gy, gx = _f32(gy), _f32(gx).copy()
+    dims = list(dims) + [1] * (len(perm) - len(dims))
+    d, nd = _dims(dims)
+    pm, _ = _ids(perm)
+    lib().ref_permute_dims_bw(_p(gy), d, nd, pm, bs, _p(gx))
+    return gx
+
+
+def flip_fw(x, dims, batch, dim):
+    x = _f32(x)
+    d, depth = _dims(dims)
+    y = np.empty_like(x)
+    lib().ref_flip(_p(x), d, depth, batch, dim, 0, _p(y))
+    return y
+
+
+def flip_bw(gy, gx, dims, batch, dim):
+    gy, gx = _f32(gy), _f32(gx).copy()
+    d, depth = _dims(dims)
+    lib().ref_flip(_p(gy), d, depth, batch, dim, 1, _p(gx))
+    return gx
+
+
+def reduce_fw(op, x, dims, batch, dim):
+    x = _f32(x)
+    assert x.size == _vol(dims) * batch
+    d, depth = _dims(dims)
+    y = np.empty(x.size // _dim(dims, dim), dtype=np.float32)
+    _ok(lib().ref_reduce_fw(REDUCE_OPS.index(op), _p(x), d, depth, batch, dim, _p(y)), op)
+    return y
+
+
+def extremum_bw(x, y, gy, gx, dims, batch, dim):
+    x, y, gy, gx = _f32(x), _f32(y), _f32(gy), _f32(gx).copy()
+    d, depth = _dims(dims)
+    lib().ref_extremum_bw(_p(x), _p(y), _p(gy), d, depth, batch, dim, _p(gx))
+    return gx
+
+
+def arg_extremum(op, x, dims, batch, dim):
+    x = _f32(x)
+    d, depth = _dims(dims)
+    n = x.size // _dim(dims, dim)
+    out = (_U * max(1, n))()
+    lib().ref_arg_extremum(1 if op == "max" else 0, _p(x), d, depth, batch, dim, out)
+    return np.array(out[:n], dtype=np.uint32)
+
+
+def broadcast_fw(x, dims, batch, dim, size):
+    x = _f32(x)
+    d, depth = _dims(dims)
+    y = np.empty(x.size * size, dtype=np.float32)
+    lib().ref_broadcast_fw(_p(x), d, depth, batch, dim, size, _p(y))
     return y

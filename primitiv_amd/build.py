@@ -16,6 +16,8 @@ SOURCES = [
     "phip_elementwise.hip",
     "phip_pointwise_unary.hip",
     "phip_pointwise_binary.hip",
+    "phip_indexing.hip",
+    "phip_reduce.hip",
     "phip_gemm_f32.hip",
     "phip_gemm_f32_direct.hip",
     "phip_gemm_f32_lds.hip",

@@ -32,6 +32,8 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_elementwise.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_pointwise_unary.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_pointwise_binary.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_indexing.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_reduce.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_direct.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip
