@@ -47,6 +47,7 @@ _sz = ctypes.c_size_t
 _f = ctypes.c_float
 _int = ctypes.c_int
 _pp = ctypes.POINTER(ctypes.c_void_p)
+_ids = ctypes.POINTER(ctypes.c_uint32)   # host array of indices / extents
 
 # name -> argument types; every function returns int unless listed in _RESTYPES
 SIGNATURES = {
@@ -118,6 +119,51 @@ SIGNATURES = {
     "phip_inplace_subtract_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
     "phip_inplace_multiply_const_bf16": [_vp, _f, _vp, _sz],
     "phip_identity_bf16": [_vp, _vp, _u32],
+    "phip_copy_rows_f32": [_vp, _vp, _vp, _u32, _u32, _u64, _u64, _u32, _u64, _u64, _int],
+    "phip_pick_fw_f32": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_pick_bw_f32": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_batch_pick_fw_f32": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_batch_pick_bw_f32": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_transpose_fw_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_transpose_bw_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_permute_dims_fw_f32": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_permute_dims_bw_f32": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_flip_fw_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_flip_bw_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_broadcast_fw_f32": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_reduce_fw_f32": [_vp, _int, _vp, _vp, _u32, _u32, _u32],
+    "phip_extremum_bw_f32": [_vp, _int, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_arg_extremum_f32": [_vp, _int, _vp, _ids, _u32, _u32, _u32],
+    "phip_copy_rows_f16": [_vp, _vp, _vp, _u32, _u32, _u64, _u64, _u32, _u64, _u64, _int],
+    "phip_pick_fw_f16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_pick_bw_f16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_batch_pick_fw_f16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_batch_pick_bw_f16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_transpose_fw_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_transpose_bw_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_permute_dims_fw_f16": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_permute_dims_bw_f16": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_flip_fw_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_flip_bw_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_broadcast_fw_f16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_reduce_fw_f16": [_vp, _int, _vp, _vp, _u32, _u32, _u32],
+    "phip_extremum_bw_f16": [_vp, _int, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_arg_extremum_f16": [_vp, _int, _vp, _ids, _u32, _u32, _u32],
+    "phip_copy_rows_bf16": [_vp, _vp, _vp, _u32, _u32, _u64, _u64, _u32, _u64, _u64, _int],
+    "phip_pick_fw_bf16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_pick_bw_bf16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_batch_pick_fw_bf16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_batch_pick_bw_bf16": [_vp, _vp, _ids, _u32, _vp, _u32, _u32],
+    "phip_transpose_fw_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_transpose_bw_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_permute_dims_fw_bf16": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_permute_dims_bw_bf16": [_vp, _vp, _vp, _u32, _ids, _ids, _u32],
+    "phip_flip_fw_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_flip_bw_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_broadcast_fw_bf16": [_vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_reduce_fw_bf16": [_vp, _int, _vp, _vp, _u32, _u32, _u32],
+    "phip_extremum_bw_bf16": [_vp, _int, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "phip_arg_extremum_bf16": [_vp, _int, _vp, _ids, _u32, _u32, _u32],
     "phip_matmul_fw_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_f16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_bf16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],

@@ -72,6 +72,24 @@ class Shape:
     def resize_batch(self, batch):
         return Shape(self._dims, batch)
 
+    def lower_volume(self, dim):
+        # shape.h:100-104: product of the dimensions below `dim`
+        v = 1
+        for d in self._dims[:dim]:
+            v *= d
+        return v
+
+    def resize_dim(self, dim, m):
+        # shape.cc: the same shape with dimension `dim` set to m
+        dims = list(self._dims) + [1] * max(0, dim + 1 - len(self._dims))
+        dims[dim] = m
+        return Shape(dims, self._batch)
+
+    def has_same_loo_dims(self, rhs, dim):
+        # shape.cc: equal in every dimension except `dim` ("leave one out")
+        depth = max(len(self._dims), len(rhs._dims))
+        return all(self[i] == rhs[i] for i in range(depth) if i != dim)
+
     def to_string(self):
         return "[%s]x%d" % (",".join(str(d) for d in self._dims), self._batch)
 
@@ -106,6 +124,91 @@ class shape_ops:
     @staticmethod
     def batch_sum(x):
         return x.resize_batch(1)
+
+    @staticmethod
+    def slice(x, dim, lower, upper):
+        # shape_ops.cc:43-53
+        if lower >= upper or upper > x[dim]:
+            raise Error("Invalid slice operation. shape: %s, dim: %d, lower: %d, upper: %d"
+                        % (x.to_string(), dim, lower, upper))
+        return x if dim >= x.depth() else x.resize_dim(dim, upper - lower)
+
+    @staticmethod
+    def concat(xs, dim):
+        # shape_ops.cc:62-87
+        if not xs:
+            raise Error("No tensors to be concatenated.")
+        s0, total = xs[0], xs[0][dim]
+        for s in xs[1:]:
+            if not s0.has_same_loo_dims(s, dim) or not s0.has_compatible_batch(s):
+                raise Error("Invalid shapes to concatenate: " + ", ".join(x.to_string() for x in xs))
+            if not s0.has_batch():
+                s0 = s0.resize_batch(s.batch())
+            total += s[dim]
+        return s0.resize_dim(dim, total)
+
+    @staticmethod
+    def broadcast(x, dim, size):
+        # shape_ops.cc:89-96
+        if x[dim] != 1 or size == 0:
+            raise Error("Invalid broadcasting. x: %s, dim: %d, size: %d" % (x.to_string(), dim, size))
+        return x.resize_dim(dim, size)
+
+    @staticmethod
+    def pick(x, ids, dim):
+        # shape_ops.cc:98-118
+        n, bi = x[dim], len(ids)
+        if bi == 0 or (x.batch() != bi and x.has_batch() and bi > 1):
+            raise Error("Invalid IDs to pick. shape: %s, ids.size(): %d" % (x.to_string(), bi))
+        for i, v in enumerate(ids):
+            if v >= n:
+                raise Error("Invalid IDs to pick. shape: %s, ids[%d]: %d" % (x.to_string(), i, v))
+        return x.resize_dim(dim, 1).resize_batch(max(x.batch(), bi))
+
+    @staticmethod
+    def transpose(x):
+        # shape_ops.cc:120-125
+        if not x.is_matrix():
+            raise Error("Invalid shape to transpose: " + x.to_string())
+        return Shape([x[1], x[0]], x.batch())
+
+    @staticmethod
+    def permute_dims(x, perm):
+        # shape_ops.cc:127-152
+        if len(perm) < x.depth():
+            raise Error("Invalid perm to permute. shape: %s, perm.size(): %d" % (x.to_string(), len(perm)))
+        if sorted(perm) != list(range(len(perm))):
+            raise Error("Invalid perm to permute. shape: %s, perm: %s" % (x.to_string(), list(perm)))
+        return Shape([x[p] for p in perm], x.batch())
+
+    @staticmethod
+    def batch_pick(x, ids):
+        # shape_ops.cc:216-233
+        if len(ids) == 0:
+            raise Error("Invalid IDs to pick. shape: %s, ids.size(): 0" % x.to_string())
+        for i, v in enumerate(ids):
+            if v >= x.batch():
+                raise Error("Invalid IDs to pick. shape: %s, ids[%d]: %d" % (x.to_string(), i, v))
+        return x.resize_batch(len(ids))
+
+    @staticmethod
+    def batch_slice(x, lower, upper):
+        # shape_ops.cc:235-243
+        if lower >= upper or upper > x.batch():
+            raise Error("Invalid batch_slice operation. shape: %s, lower: %d, upper: %d"
+                        % (x.to_string(), lower, upper))
+        return x.resize_batch(upper - lower)
+
+    @staticmethod
+    def batch_concat(xs):
+        # shape_ops.cc:252-274
+        if not xs:
+            raise Error("No tensors to be concatenated.")
+        for s in xs[1:]:
+            if not xs[0].has_same_dims(s):
+                raise Error("Invalid shapes to concatenate minibatches: "
+                            + ", ".join(x.to_string() for x in xs))
+        return xs[0].resize_batch(sum(s.batch() for s in xs))
 
     @staticmethod
     def elementwise(a, b):
@@ -520,6 +623,259 @@ class HIP:
             raise Error("Invalid size of the identity matrix. size: 0")
         y = self.new_raw_tensor(Shape([size, size]))
         _lib.call("phip_identity_" + self._SUFFIX, self._ctx, y.mutable_handle(), size)
+        return y
+
+    # -- moving and reducing along one dimension --------------------------------
+    REDUCE_OPS = ("sum", "logsumexp", "max", "min")
+
+    @staticmethod
+    def _u32(values):
+        values = [int(v) for v in values]
+        return (ctypes.c_uint32 * max(1, len(values)))(*values), len(values)
+
+    def _copy_rows(self, src, dst, span, rows, ss, ds, bs, sbs, dbs, accumulate):
+        _lib.call("phip_copy_rows_" + self._SUFFIX, self._ctx, src, dst, span, rows, ss, ds, bs, sbs, dbs,
+                  int(accumulate))
+
+    def _at(self, ptr, elements):
+        """Device address `elements` elements past ptr."""
+        return ptr + elements * self._ITEMSIZE
+
+    def slice_fw(self, x, dim, lower, upper):
+        # device.cc:157-164; devices/cuda/ops/slice.cu:26-37
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.slice(x.shape(), dim, lower, upper))
+        sx, sy = x.shape(), y.shape()
+        base = sy.lower_volume(dim)
+        span, skip = base * sy[dim], base * sx[dim]
+        self._copy_rows(self._at(x.handle(), base * lower), y.mutable_handle(), span, sy.size() // span,
+                        skip, span, 1, 0, 0, False)
+        return y
+
+    def slice_bw(self, gy, dim, offset, gx):
+        # device.cc:195-211; devices/cuda/ops/slice.cu:39-55
+        self._check_device(gy)
+        self._check_device(gx)
+        sy, sx = gy.shape(), gx.shape()
+        if (not sy.has_same_loo_dims(sx, dim) or not sy.has_compatible_batch(sx)
+                or offset + sy[dim] > sx[dim]):
+            raise Error("Attempted to add gradients with shape %s, dim %d, offset %d to shape%s."
+                        % (sy.to_string(), dim, offset, sx.to_string()))
+        if dim >= sx.depth():
+            return self.inplace_add(gy, gx)
+        base = sx.lower_volume(dim)
+        span, skip = base * sy[dim], base * sx[dim]
+        pgx = gx.mutable_handle()
+        self._copy_rows(gy.handle(), self._at(pgx, base * offset), span, sx.volume() // skip, span, skip,
+                        max(sx.batch(), sy.batch()), sy.volume() if sy.has_batch() else 0,
+                        sx.volume() if sx.has_batch() else 0, True)
+
+    def concat_fw(self, xs, dim):
+        # device.cc:166-179; devices/cuda/ops/concat.cu:20-40
+        if not xs:
+            raise Error("No tensors to concat.")
+        for x in xs:
+            self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.concat([x.shape() for x in xs], dim))
+        sy = y.shape()
+        base = sy.lower_volume(dim)
+        skip = base * sy[dim]
+        repeat = sy.volume() // skip
+        py, offset = y.mutable_handle(), 0
+        for x in xs:
+            span = base * x.shape()[dim]
+            self._copy_rows(x.handle(), self._at(py, offset), span, repeat, span, skip, sy.batch(),
+                            x.shape().volume() if x.shape().has_batch() else 0, sy.volume(), False)
+            offset += span
+        return y
+
+    def pick_fw(self, x, ids, dim):
+        # device.cc:150-155
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.pick(x.shape(), ids, dim))
+        sx = x.shape()
+        base = sx.lower_volume(dim)
+        arr, n = self._u32(ids)
+        _lib.call("phip_pick_fw_" + self._SUFFIX, self._ctx, x.handle(), arr, n, y.mutable_handle(), base,
+                  sx[dim], sx.volume() // (base * sx[dim]), sx.batch(), y.shape().batch())
+        return y
+
+    def pick_bw(self, gy, ids, dim, gx):
+        # device.cc:181-193
+        self._check_device(gy)
+        self._check_device(gx)
+        sx = gx.shape()
+        sy = shape_ops.pick(sx, ids, dim)
+        if gy.shape() != sy:
+            raise Error("Shape mismatched. gy.shape(): %s != expected shape: %s"
+                        % (gy.shape().to_string(), sy.to_string()))
+        base = sx.lower_volume(dim)
+        arr, n = self._u32(ids)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_pick_bw_" + self._SUFFIX, self._ctx, gy.handle(), arr, n, pgx, base, sx[dim],
+                  sx.volume() // (base * sx[dim]), sx.batch(), sy.batch())
+
+    def batch_pick_fw(self, x, ids):
+        # device.cc:616-622
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.batch_pick(x.shape(), ids))
+        arr, n = self._u32(ids)
+        _lib.call("phip_batch_pick_fw_" + self._SUFFIX, self._ctx, x.handle(), arr, n, y.mutable_handle(),
+                  x.shape().volume(), x.shape().batch())
+        return y
+
+    def batch_pick_bw(self, gy, ids, gx):
+        # device.cc:653-664
+        self._check_device(gy)
+        self._check_device(gx)
+        sy = shape_ops.batch_pick(gx.shape(), ids)
+        if gy.shape() != sy:
+            raise Error("Shape mismatched. gy.shape(): %s != expected shape: %s"
+                        % (gy.shape().to_string(), sy.to_string()))
+        arr, n = self._u32(ids)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_batch_pick_bw_" + self._SUFFIX, self._ctx, gy.handle(), arr, n, pgx,
+                  gx.shape().volume(), gx.shape().batch())
+
+    def batch_slice_fw(self, x, lower, upper):
+        # device.cc:624-630
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.batch_slice(x.shape(), lower, upper))
+        vol = y.shape().volume()
+        self._copy_rows(self._at(x.handle(), vol * lower), y.mutable_handle(), vol, y.shape().batch(), vol, vol,
+                        1, 0, 0, False)
+        return y
+
+    def batch_slice_bw(self, gy, offset, gx):
+        # device.cc:666-679
+        self._check_device(gy)
+        self._check_device(gx)
+        sy, sx = gy.shape(), gx.shape()
+        if not sy.has_same_dims(sx) or offset + sy.batch() > sx.batch():
+            raise Error("Attempted to add gradients with shape %s, batch offset %d to shape%s."
+                        % (sy.to_string(), offset, sx.to_string()))
+        vol = sy.volume()
+        pgx = gx.mutable_handle()
+        self._copy_rows(gy.handle(), self._at(pgx, vol * offset), vol, sy.batch(), vol, vol, 1, 0, 0, True)
+
+    def batch_concat_fw(self, xs):
+        # device.cc:632-644
+        if not xs:
+            raise Error("No tensors to concat.")
+        for x in xs:
+            self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.batch_concat([x.shape() for x in xs]))
+        vol = y.shape().volume()
+        py, offset = y.mutable_handle(), 0
+        for x in xs:
+            self._copy_rows(x.handle(), self._at(py, offset), vol, x.shape().batch(), vol, vol, 1, 0, 0, False)
+            offset += x.shape().size()
+        return y
+
+    def transpose_fw(self, x):
+        # DEV_FW_X(transpose, shape_ops::transpose), device.cc:314
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.transpose(x.shape()))
+        _lib.call("phip_transpose_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(), x.shape()[0],
+                  x.shape()[1], x.shape().batch())
+        return y
+
+    def transpose_bw(self, x, y, gy, gx):
+        # DEV_BW_X(transpose, shape_ops::transpose), device.cc:334
+        for t in (x, y, gy, gx):
+            self._check_device(t)
+        if (x.shape() != gx.shape() or y.shape() != gy.shape()
+                or y.shape() != shape_ops.transpose(x.shape())):
+            raise Error("Shape mismatched at transpose_bw. x.shape: %s, y.shape: %s, gy.shape: %s, gx.shape: %s"
+                        % tuple(t.shape().to_string() for t in (x, y, gy, gx)))
+        pgx = gx.mutable_handle()
+        _lib.call("phip_transpose_bw_" + self._SUFFIX, self._ctx, gy.handle(), pgx, gx.shape()[0],
+                  gx.shape()[1], gx.shape().batch())
+
+    def permute_dims_fw(self, x, perm):
+        # device.cc:316-322
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.permute_dims(x.shape(), perm))
+        dims, n = self._u32([x.shape()[i] for i in range(len(perm))])
+        pm, _ = self._u32(perm)
+        _lib.call("phip_permute_dims_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(), n, dims, pm,
+                  x.shape().batch())
+        return y
+
+    def permute_dims_bw(self, x, y, gy, perm, gx):
+        # device.cc:336-354
+        for t in (x, y, gy, gx):
+            self._check_device(t)
+        sy = shape_ops.permute_dims(x.shape(), perm)
+        if y.shape() != sy or gy.shape() != sy or gx.shape() != x.shape():
+            raise Error("Shape mismatched at permute_dims_bw. x.shape: %s, y.shape: %s, gy.shape: %s, gx.shape: %s"
+                        % tuple(t.shape().to_string() for t in (x, y, gy, gx)))
+        dims, n = self._u32([x.shape()[i] for i in range(len(perm))])
+        pm, _ = self._u32(perm)
+        pgx = gx.mutable_handle()
+        _lib.call("phip_permute_dims_bw_" + self._SUFFIX, self._ctx, gy.handle(), pgx, n, dims, pm,
+                  x.shape().batch())
+
+    def _around(self, s, dim):
+        """(base, n, outer) of shape s seen around dimension dim."""
+        base = s.lower_volume(dim)
+        return base, s[dim], s.size() // (base * s[dim])
+
+    def flip_fw(self, x, dim):
+        # device.cc:530-535
+        self._check_device(x)
+        y = self.new_raw_tensor(x.shape())
+        _lib.call("phip_flip_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(),
+                  *self._around(x.shape(), dim))
+        return y
+
+    def flip_bw(self, gy, dim, gx):
+        # device.cc:537-547
+        self._check_device(gy)
+        self._check_device(gx)
+        if gy.shape() != gx.shape():
+            raise Error("Shape mismatched. gy.shape(): %s != expected shape: %s"
+                        % (gy.shape().to_string(), gx.shape().to_string()))
+        pgx = gx.mutable_handle()
+        _lib.call("phip_flip_bw_" + self._SUFFIX, self._ctx, gy.handle(), pgx, *self._around(gx.shape(), dim))
+
+    def reduce_fw(self, op, x, dim):
+        """sum_fw / logsumexp_fw / max_fw / min_fw along dim (device.cc:549-561,597-609)."""
+        self._check_device(x)
+        y = self.new_raw_tensor(x.shape().resize_dim(dim, 1))
+        _lib.call("phip_reduce_fw_" + self._SUFFIX, self._ctx, self.REDUCE_OPS.index(op), x.handle(),
+                  y.mutable_handle(), *self._around(x.shape(), dim))
+        return y
+
+    def extremum_bw(self, op, x, y, gy, dim, gx):
+        """max_bw / min_bw (device.cc:563-595)."""
+        for t in (x, y, gy, gx):
+            self._check_device(t)
+        r = x.shape()
+        s = r.resize_dim(dim, 1)
+        if gx.shape() != r or y.shape() != s or gy.shape() != s:
+            raise Error("Shape mismatched at %s_bw(dim=%d). x.shape: %s, y.shape: %s, gy.shape: %s, gx.shape: %s"
+                        % ((op, dim) + tuple(t.shape().to_string() for t in (x, y, gy, gx))))
+        pgx = gx.mutable_handle()
+        _lib.call("phip_extremum_bw_" + self._SUFFIX, self._ctx, self.REDUCE_OPS.index(op), x.handle(),
+                  y.handle(), gy.handle(), pgx, *self._around(r, dim))
+
+    def arg_extremum(self, op, x, dim):
+        """argmax / argmin along dim as a list of indices (device.cc:56-64)."""
+        self._check_device(x)
+        base, n, outer = self._around(x.shape(), dim)
+        out = (ctypes.c_uint32 * max(1, base * outer))()
+        _lib.call("phip_arg_extremum_" + self._SUFFIX, self._ctx, self.REDUCE_OPS.index(op), x.handle(), out,
+                  base, n, outer)
+        return list(out[:base * outer])
+
+    def broadcast_fw(self, x, dim, size):
+        # device.cc:611-616
+        self._check_device(x)
+        y = self.new_raw_tensor(shape_ops.broadcast(x.shape(), dim, size))
+        base = y.shape().lower_volume(dim)
+        _lib.call("phip_broadcast_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(), base, size,
+                  x.shape().size() // base)
         return y
 
 
