@@ -3,6 +3,7 @@
 
 #include <primitiv/devices/hip/device.h>
 
+#include <algorithm>
 #include <iostream>
 #include <random>
 #include <string>
@@ -49,6 +50,28 @@ struct PointwiseAbi {
   int (*identity)(phip_ctx *, void *, std::uint32_t);
 };
 
+typedef std::uint32_t U32;
+typedef std::uint64_t U64;
+
+// The same for the operations that move or reduce along one dimension.
+struct IndexingAbi {
+  int (*copy_rows)(phip_ctx *, const void *, void *, U32, U32, U64, U64, U32, U64, U64, int);
+  int (*pick_fw)(phip_ctx *, const void *, const U32 *, U32, void *, U32, U32, U32, U32, U32);
+  int (*pick_bw)(phip_ctx *, const void *, const U32 *, U32, void *, U32, U32, U32, U32, U32);
+  int (*batch_pick_fw)(phip_ctx *, const void *, const U32 *, U32, void *, U32, U32);
+  int (*batch_pick_bw)(phip_ctx *, const void *, const U32 *, U32, void *, U32, U32);
+  int (*transpose_fw)(phip_ctx *, const void *, void *, U32, U32, U32);
+  int (*transpose_bw)(phip_ctx *, const void *, void *, U32, U32, U32);
+  int (*permute_dims_fw)(phip_ctx *, const void *, void *, U32, const U32 *, const U32 *, U32);
+  int (*permute_dims_bw)(phip_ctx *, const void *, void *, U32, const U32 *, const U32 *, U32);
+  int (*flip_fw)(phip_ctx *, const void *, void *, U32, U32, U32);
+  int (*flip_bw)(phip_ctx *, const void *, void *, U32, U32, U32);
+  int (*broadcast_fw)(phip_ctx *, const void *, void *, U32, U32, U32);
+  int (*reduce_fw)(phip_ctx *, int, const void *, void *, U32, U32, U32);
+  int (*extremum_bw)(phip_ctx *, int, const void *, const void *, const void *, void *, U32, U32, U32);
+  int (*arg_extremum)(phip_ctx *, int, const void *, U32 *, U32, U32, U32);
+};
+
 typedef const float *CF;
 typedef float *MF;
 
@@ -93,6 +116,66 @@ const PointwiseAbi &pointwise_abi(primitiv::devices::HIP::Storage s) {
     case primitiv::devices::HIP::Storage::BF16: return bf16;
     default: return f32;
   }
+}
+
+const IndexingAbi &indexing_abi(primitiv::devices::HIP::Storage s) {
+  static const IndexingAbi f32 = {
+    [](phip_ctx *c, const void *src, void *dst, U32 span, U32 rows, U64 ss, U64 ds, U32 bs, U64 sbs, U64 dbs,
+       int acc) { return ::phip_copy_rows_f32(c, CF(src), MF(dst), span, rows, ss, ds, bs, sbs, dbs, acc); },
+    [](phip_ctx *c, const void *x, const U32 *ids, U32 n_ids, void *y, U32 base, U32 n, U32 outer, U32 bx,
+       U32 bs) { return ::phip_pick_fw_f32(c, CF(x), ids, n_ids, MF(y), base, n, outer, bx, bs); },
+    [](phip_ctx *c, const void *gy, const U32 *ids, U32 n_ids, void *gx, U32 base, U32 n, U32 outer, U32 bx,
+       U32 bs) { return ::phip_pick_bw_f32(c, CF(gy), ids, n_ids, MF(gx), base, n, outer, bx, bs); },
+    [](phip_ctx *c, const void *x, const U32 *ids, U32 n_ids, void *y, U32 volume, U32 bx) {
+      return ::phip_batch_pick_fw_f32(c, CF(x), ids, n_ids, MF(y), volume, bx); },
+    [](phip_ctx *c, const void *gy, const U32 *ids, U32 n_ids, void *gx, U32 volume, U32 bx) {
+      return ::phip_batch_pick_bw_f32(c, CF(gy), ids, n_ids, MF(gx), volume, bx); },
+    [](phip_ctx *c, const void *x, void *y, U32 rows, U32 cols, U32 bs) {
+      return ::phip_transpose_fw_f32(c, CF(x), MF(y), rows, cols, bs); },
+    [](phip_ctx *c, const void *gy, void *gx, U32 rows, U32 cols, U32 bs) {
+      return ::phip_transpose_bw_f32(c, CF(gy), MF(gx), rows, cols, bs); },
+    [](phip_ctx *c, const void *x, void *y, U32 nd, const U32 *dims, const U32 *perm, U32 bs) {
+      return ::phip_permute_dims_fw_f32(c, CF(x), MF(y), nd, dims, perm, bs); },
+    [](phip_ctx *c, const void *gy, void *gx, U32 nd, const U32 *dims, const U32 *perm, U32 bs) {
+      return ::phip_permute_dims_bw_f32(c, CF(gy), MF(gx), nd, dims, perm, bs); },
+    [](phip_ctx *c, const void *x, void *y, U32 base, U32 n, U32 outer) {
+      return ::phip_flip_fw_f32(c, CF(x), MF(y), base, n, outer); },
+    [](phip_ctx *c, const void *gy, void *gx, U32 base, U32 n, U32 outer) {
+      return ::phip_flip_bw_f32(c, CF(gy), MF(gx), base, n, outer); },
+    [](phip_ctx *c, const void *x, void *y, U32 base, U32 size, U32 outer) {
+      return ::phip_broadcast_fw_f32(c, CF(x), MF(y), base, size, outer); },
+    [](phip_ctx *c, int op, const void *x, void *y, U32 base, U32 n, U32 outer) {
+      return ::phip_reduce_fw_f32(c, op, CF(x), MF(y), base, n, outer); },
+    [](phip_ctx *c, int op, const void *x, const void *y, const void *gy, void *gx, U32 base, U32 n, U32 outer) {
+      return ::phip_extremum_bw_f32(c, op, CF(x), CF(y), CF(gy), MF(gx), base, n, outer); },
+    [](phip_ctx *c, int op, const void *x, U32 *out, U32 base, U32 n, U32 outer) {
+      return ::phip_arg_extremum_f32(c, op, CF(x), out, base, n, outer); },
+  };
+  static const IndexingAbi f16 = {
+    ::phip_copy_rows_f16, ::phip_pick_fw_f16, ::phip_pick_bw_f16, ::phip_batch_pick_fw_f16,
+    ::phip_batch_pick_bw_f16, ::phip_transpose_fw_f16, ::phip_transpose_bw_f16, ::phip_permute_dims_fw_f16,
+    ::phip_permute_dims_bw_f16, ::phip_flip_fw_f16, ::phip_flip_bw_f16, ::phip_broadcast_fw_f16,
+    ::phip_reduce_fw_f16, ::phip_extremum_bw_f16, ::phip_arg_extremum_f16,
+  };
+  static const IndexingAbi bf16 = {
+    ::phip_copy_rows_bf16, ::phip_pick_fw_bf16, ::phip_pick_bw_bf16, ::phip_batch_pick_fw_bf16,
+    ::phip_batch_pick_bw_bf16, ::phip_transpose_fw_bf16, ::phip_transpose_bw_bf16, ::phip_permute_dims_fw_bf16,
+    ::phip_permute_dims_bw_bf16, ::phip_flip_fw_bf16, ::phip_flip_bw_bf16, ::phip_broadcast_fw_bf16,
+    ::phip_reduce_fw_bf16, ::phip_extremum_bw_bf16, ::phip_arg_extremum_bf16,
+  };
+  switch (s) {
+    case primitiv::devices::HIP::Storage::F16: return f16;
+    case primitiv::devices::HIP::Storage::BF16: return bf16;
+    default: return f32;
+  }
+}
+
+// Address `elements` elements past p for a storage type.
+inline const void *advance(const void *p, std::size_t elements, primitiv::devices::HIP::Storage s) {
+  return static_cast<const char *>(p) + elements * (s == primitiv::devices::HIP::Storage::F32 ? 4 : 2);
+}
+inline void *advance(void *p, std::size_t elements, primitiv::devices::HIP::Storage s) {
+  return static_cast<char *>(p) + elements * (s == primitiv::devices::HIP::Storage::F32 ? 4 : 2);
 }
 
 }  // namespace
@@ -327,6 +410,197 @@ void HIP::inplace_subtract_impl(const Tensor &x, Tensor &y) {
 void HIP::inplace_multiply_const_impl(float k, Tensor &x) {
   PHIP_CALL(pointwise_abi(storage_).inplace_multiply_const(ctx_, k, get_mutable_handle(x), x.shape().size()));
 }
+
+// ---- moving and reducing along one dimension -------------------------------------
+// A tensor is seen around `dim` as [outer][n][base] (base = lower_volume(dim));
+// the offsets handed to libphip are those of the reference's kernels
+// (primitiv/devices/cuda/ops/{slice,concat,pick,batch_pick,batch_slice,
+// batch_concat,transpose,permute_dims,flip,sum,logsumexp,max,min,argmax,
+// argmin,broadcast}.cu).
+
+void HIP::slice_fw_impl(const Tensor &x, std::uint32_t dim, std::uint32_t offset, Tensor &y) {
+  const std::uint32_t base = y.shape().lower_volume(dim);
+  const std::uint32_t span = base * y.shape()[dim];
+  const std::uint32_t skip = base * x.shape()[dim];
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).copy_rows(
+      ctx_, advance(get_handle(x), static_cast<std::size_t>(base) * offset, storage_), py,
+      span, y.shape().size() / span, skip, span, 1, 0, 0, 0));
+}
+
+void HIP::slice_bw_impl(const Tensor &gy, std::uint32_t dim, std::uint32_t offset, Tensor &gx) {
+  const Shape &sx = gx.shape();
+  const Shape &sy = gy.shape();
+  const std::uint32_t base = sx.lower_volume(dim);
+  const std::uint32_t span = base * sy[dim];
+  const std::uint32_t skip = base * sx[dim];
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).copy_rows(
+      ctx_, get_handle(gy), advance(pgx, static_cast<std::size_t>(base) * offset, storage_),
+      span, sx.volume() / skip, span, skip, std::max(sx.batch(), sy.batch()),
+      sy.has_batch() ? sy.volume() : 0, sx.has_batch() ? sx.volume() : 0, 1));
+}
+
+void HIP::concat_fw_impl(const std::vector<const Tensor *> &xs, std::uint32_t dim, Tensor &y) {
+  const Shape &sy = y.shape();
+  const std::uint32_t base = sy.lower_volume(dim);
+  const std::uint32_t skip = base * sy[dim];
+  const std::uint32_t repeat = sy.volume() / skip;
+  void *py = get_mutable_handle(y);
+  std::size_t offset = 0;
+  for (const Tensor *x : xs) {
+    const std::uint32_t span = base * x->shape()[dim];
+    PHIP_CALL(indexing_abi(storage_).copy_rows(
+        ctx_, get_handle(*x), advance(py, offset, storage_), span, repeat, span, skip, sy.batch(),
+        x->shape().has_batch() ? x->shape().volume() : 0, sy.volume(), 0));
+    offset += span;
+  }
+}
+
+void HIP::pick_fw_impl(
+    const Tensor &x, const std::vector<std::uint32_t> &ids, std::uint32_t dim, Tensor &y) {
+  const Shape &sx = x.shape();
+  const std::uint32_t base = sx.lower_volume(dim);
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).pick_fw(
+      ctx_, get_handle(x), ids.data(), ids.size(), py, base, sx[dim], sx.volume() / (base * sx[dim]),
+      sx.batch(), y.shape().batch()));
+}
+
+void HIP::pick_bw_impl(
+    const Tensor &gy, const std::vector<std::uint32_t> &ids, std::uint32_t dim, Tensor &gx) {
+  const Shape &sx = gx.shape();
+  const std::uint32_t base = sx.lower_volume(dim);
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).pick_bw(
+      ctx_, get_handle(gy), ids.data(), ids.size(), pgx, base, sx[dim], sx.volume() / (base * sx[dim]),
+      sx.batch(), gy.shape().batch()));
+}
+
+void HIP::batch_pick_fw_impl(const Tensor &x, const std::vector<std::uint32_t> &ids, Tensor &y) {
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).batch_pick_fw(
+      ctx_, get_handle(x), ids.data(), ids.size(), py, x.shape().volume(), x.shape().batch()));
+}
+
+void HIP::batch_pick_bw_impl(const Tensor &gy, const std::vector<std::uint32_t> &ids, Tensor &gx) {
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).batch_pick_bw(
+      ctx_, get_handle(gy), ids.data(), ids.size(), pgx, gx.shape().volume(), gx.shape().batch()));
+}
+
+void HIP::batch_slice_fw_impl(const Tensor &x, std::uint32_t offset, Tensor &y) {
+  const std::uint32_t volume = y.shape().volume();
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).copy_rows(
+      ctx_, advance(get_handle(x), static_cast<std::size_t>(volume) * offset, storage_), py,
+      volume, y.shape().batch(), volume, volume, 1, 0, 0, 0));
+}
+
+void HIP::batch_slice_bw_impl(const Tensor &gy, std::uint32_t offset, Tensor &gx) {
+  const std::uint32_t volume = gy.shape().volume();
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).copy_rows(
+      ctx_, get_handle(gy), advance(pgx, static_cast<std::size_t>(volume) * offset, storage_),
+      volume, gy.shape().batch(), volume, volume, 1, 0, 0, 1));
+}
+
+void HIP::batch_concat_fw_impl(const std::vector<const Tensor *> &xs, Tensor &y) {
+  const std::uint32_t volume = y.shape().volume();
+  void *py = get_mutable_handle(y);
+  std::size_t offset = 0;
+  for (const Tensor *x : xs) {
+    PHIP_CALL(indexing_abi(storage_).copy_rows(
+        ctx_, get_handle(*x), advance(py, offset, storage_), volume, x->shape().batch(), volume, volume,
+        1, 0, 0, 0));
+    offset += x->shape().size();
+  }
+}
+
+void HIP::transpose_fw_impl(const Tensor &x, Tensor &y) {
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).transpose_fw(
+      ctx_, get_handle(x), py, x.shape()[0], x.shape()[1], x.shape().batch()));
+}
+
+void HIP::transpose_bw_impl(const Tensor &, const Tensor &, const Tensor &gy, Tensor &gx) {
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).transpose_bw(
+      ctx_, get_handle(gy), pgx, gx.shape()[0], gx.shape()[1], gx.shape().batch()));
+}
+
+void HIP::permute_dims_fw_impl(const Tensor &x, const std::vector<std::uint32_t> &perm, Tensor &y) {
+  std::vector<std::uint32_t> dims(perm.size());
+  for (std::size_t i = 0; i < perm.size(); ++i) dims[i] = x.shape()[i];
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).permute_dims_fw(
+      ctx_, get_handle(x), py, perm.size(), dims.data(), perm.data(), x.shape().batch()));
+}
+
+void HIP::permute_dims_bw_impl(
+    const Tensor &, const Tensor &, const Tensor &gy, const std::vector<std::uint32_t> &perm, Tensor &gx) {
+  std::vector<std::uint32_t> dims(perm.size());
+  for (std::size_t i = 0; i < perm.size(); ++i) dims[i] = gx.shape()[i];
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).permute_dims_bw(
+      ctx_, get_handle(gy), pgx, perm.size(), dims.data(), perm.data(), gx.shape().batch()));
+}
+
+void HIP::flip_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) {
+  const Shape &s = x.shape();
+  const std::uint32_t base = s.lower_volume(dim), n = s[dim];
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).flip_fw(ctx_, get_handle(x), py, base, n, s.size() / (base * n)));
+}
+
+void HIP::flip_bw_impl(const Tensor &gy, std::uint32_t dim, Tensor &gx) {
+  const Shape &s = gx.shape();
+  const std::uint32_t base = s.lower_volume(dim), n = s[dim];
+  void *pgx = get_mutable_handle(gx);
+  PHIP_CALL(indexing_abi(storage_).flip_bw(ctx_, get_handle(gy), pgx, base, n, s.size() / (base * n)));
+}
+
+void HIP::broadcast_fw_impl(const Tensor &x, std::uint32_t dim, std::uint32_t size, Tensor &y) {
+  const std::uint32_t base = y.shape().lower_volume(dim);
+  void *py = get_mutable_handle(y);
+  PHIP_CALL(indexing_abi(storage_).broadcast_fw(ctx_, get_handle(x), py, base, size, x.shape().size() / base));
+}
+
+#define PHIP_DEF_REDUCE(name, code) \
+void HIP::name##_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) { \
+  const Shape &s = x.shape(); \
+  const std::uint32_t base = s.lower_volume(dim), n = s[dim]; \
+  void *py = get_mutable_handle(y); \
+  PHIP_CALL(indexing_abi(storage_).reduce_fw(ctx_, code, get_handle(x), py, base, n, s.size() / (base * n))); \
+}
+
+#define PHIP_DEF_EXTREMUM(name, code) \
+void HIP::name##_bw_impl( \
+    const Tensor &x, const Tensor &y, const Tensor &gy, std::uint32_t dim, Tensor &gx) { \
+  const Shape &s = x.shape(); \
+  const std::uint32_t base = s.lower_volume(dim), n = s[dim]; \
+  void *pgx = get_mutable_handle(gx); \
+  PHIP_CALL(indexing_abi(storage_).extremum_bw( \
+      ctx_, code, get_handle(x), get_handle(y), get_handle(gy), pgx, base, n, s.size() / (base * n))); \
+} \
+std::vector<std::uint32_t> HIP::arg##name##_impl(const Tensor &x, std::uint32_t dim) { \
+  const Shape &s = x.shape(); \
+  const std::uint32_t base = s.lower_volume(dim), n = s[dim]; \
+  std::vector<std::uint32_t> ret(s.size() / n); \
+  PHIP_CALL(indexing_abi(storage_).arg_extremum( \
+      ctx_, code, get_handle(x), ret.data(), base, n, s.size() / (base * n))); \
+  return ret; \
+}
+
+PHIP_DEF_REDUCE(sum, PHIP_SUM)
+PHIP_DEF_REDUCE(logsumexp, PHIP_LOGSUMEXP)
+PHIP_DEF_REDUCE(max, PHIP_MAX)
+PHIP_DEF_REDUCE(min, PHIP_MIN)
+PHIP_DEF_EXTREMUM(max, PHIP_MAX)
+PHIP_DEF_EXTREMUM(min, PHIP_MIN)
+
+#undef PHIP_DEF_REDUCE
+#undef PHIP_DEF_EXTREMUM
 
 // ---- elementwise families ------------------------------------------------------
 // One definition per Device virtual; the libphip operation code names the

@@ -79,6 +79,34 @@ private:
   void inplace_subtract_impl(const Tensor &x, Tensor &y) override;
   void inplace_multiply_const_impl(float k, Tensor &x) override;
 
+  // moving and reducing along one dimension
+  std::vector<std::uint32_t> argmax_impl(const Tensor &x, std::uint32_t dim) override;
+  std::vector<std::uint32_t> argmin_impl(const Tensor &x, std::uint32_t dim) override;
+  void pick_fw_impl(const Tensor &x, const std::vector<std::uint32_t> &ids, std::uint32_t dim, Tensor &y) override;
+  void slice_fw_impl(const Tensor &x, std::uint32_t dim, std::uint32_t offset, Tensor &y) override;
+  void concat_fw_impl(const std::vector<const Tensor *> &xs, std::uint32_t dim, Tensor &y) override;
+  void pick_bw_impl(const Tensor &gy, const std::vector<std::uint32_t> &ids, std::uint32_t dim, Tensor &gx) override;
+  void slice_bw_impl(const Tensor &gy, std::uint32_t dim, std::uint32_t offset, Tensor &gx) override;
+  void transpose_fw_impl(const Tensor &x, Tensor &y) override;
+  void transpose_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, Tensor &gx) override;
+  void permute_dims_fw_impl(const Tensor &x, const std::vector<std::uint32_t> &perm, Tensor &y) override;
+  void permute_dims_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy,
+                            const std::vector<std::uint32_t> &perm, Tensor &gx) override;
+  void flip_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) override;
+  void flip_bw_impl(const Tensor &gy, std::uint32_t dim, Tensor &gx) override;
+  void max_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) override;
+  void min_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) override;
+  void sum_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) override;
+  void logsumexp_fw_impl(const Tensor &x, std::uint32_t dim, Tensor &y) override;
+  void max_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, std::uint32_t dim, Tensor &gx) override;
+  void min_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, std::uint32_t dim, Tensor &gx) override;
+  void broadcast_fw_impl(const Tensor &x, std::uint32_t dim, std::uint32_t size, Tensor &y) override;
+  void batch_pick_fw_impl(const Tensor &x, const std::vector<std::uint32_t> &ids, Tensor &y) override;
+  void batch_slice_fw_impl(const Tensor &x, std::uint32_t offset, Tensor &y) override;
+  void batch_concat_fw_impl(const std::vector<const Tensor *> &xs, Tensor &y) override;
+  void batch_pick_bw_impl(const Tensor &gy, const std::vector<std::uint32_t> &ids, Tensor &gx) override;
+  void batch_slice_bw_impl(const Tensor &gy, std::uint32_t offset, Tensor &gx) override;
+
   // elementwise families (libphip operation codes select the member)
 #define PHIP_DECL_X(name) \
   void name##_fw_impl(const Tensor &x, Tensor &y) override; \
@@ -112,45 +140,11 @@ private:
   // ---- not implemented in this backend -------------------------------------
   [[noreturn]] static void unsupported(const char *op);
 
-#define PHIP_NI_X(name) \
-  void name##_impl(const Tensor &, Tensor &) override { unsupported(#name); }
-#define PHIP_NI_X_BW(name) \
-  void name##_impl(const Tensor &, const Tensor &, const Tensor &, Tensor &) override { unsupported(#name); }
-#define PHIP_NI_DIM(name) \
-  void name##_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported(#name "_fw"); }
-#define PHIP_NI_DIM_BW(name) \
-  void name##_bw_impl(const Tensor &, const Tensor &, const Tensor &, std::uint32_t, Tensor &) override { unsupported(#name "_bw"); }
 #define PHIP_NI_RANDOM(name) \
   void random_##name##_impl(float, float, Tensor &) override { unsupported("random_" #name); }
 
-  std::vector<std::uint32_t> argmax_impl(const Tensor &, std::uint32_t) override { unsupported("argmax"); }
-  std::vector<std::uint32_t> argmin_impl(const Tensor &, std::uint32_t) override { unsupported("argmin"); }
   void random_bernoulli_impl(float, Tensor &) override { unsupported("random_bernoulli"); }
   PHIP_NI_RANDOM(uniform) PHIP_NI_RANDOM(normal) PHIP_NI_RANDOM(log_normal)
-
-  void pick_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, std::uint32_t, Tensor &) override { unsupported("pick_fw"); }
-  void slice_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("slice_fw"); }
-  void concat_fw_impl(const std::vector<const Tensor *> &, std::uint32_t, Tensor &) override { unsupported("concat_fw"); }
-  void pick_bw_impl(const Tensor &, const std::vector<std::uint32_t> &, std::uint32_t, Tensor &) override { unsupported("pick_bw"); }
-  void slice_bw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("slice_bw"); }
-
-  PHIP_NI_X(transpose_fw)
-  void permute_dims_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_fw"); }
-  void flip_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_fw"); }
-
-  PHIP_NI_X_BW(transpose_bw)
-  void permute_dims_bw_impl(const Tensor &, const Tensor &, const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("permute_dims_bw"); }
-  void flip_bw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("flip_bw"); }
-
-  PHIP_NI_DIM(max) PHIP_NI_DIM(min) PHIP_NI_DIM(sum) PHIP_NI_DIM(logsumexp)
-  PHIP_NI_DIM_BW(max) PHIP_NI_DIM_BW(min)
-  void broadcast_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("broadcast_fw"); }
-
-  void batch_pick_fw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("batch_pick_fw"); }
-  void batch_slice_fw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("batch_slice_fw"); }
-  void batch_concat_fw_impl(const std::vector<const Tensor *> &, Tensor &) override { unsupported("batch_concat_fw"); }
-  void batch_pick_bw_impl(const Tensor &, const std::vector<std::uint32_t> &, Tensor &) override { unsupported("batch_pick_bw"); }
-  void batch_slice_bw_impl(const Tensor &, std::uint32_t, Tensor &) override { unsupported("batch_slice_bw"); }
 
   void conv2d_fw_impl(const Tensor &, const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t,
                       std::uint32_t, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("conv2d_fw"); }
@@ -163,10 +157,6 @@ private:
                           std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
                           Tensor &) override { unsupported("max_pool2d_bw"); }
 
-#undef PHIP_NI_X
-#undef PHIP_NI_X_BW
-#undef PHIP_NI_DIM
-#undef PHIP_NI_DIM_BW
 #undef PHIP_NI_RANDOM
 
   // Bytes of device storage for `n` elements (16-bit storage rounds the
