@@ -460,6 +460,39 @@ int phip_arg_extremum_f16(phip_ctx *ctx, int op, const void *x, uint32_t *host_o
 int phip_arg_extremum_bf16(phip_ctx *ctx, int op, const void *x, uint32_t *host_out,
                           uint32_t base, uint32_t n, uint32_t outer);
 
+/* ---- random tensors ----------------------------------------------------------
+ * Reference: random_bernoulli_impl, random_uniform_impl, random_normal_impl,
+ * random_log_normal_impl (primitiv/core/device.h:381-384; primitiv/devices/
+ * cuda/ops/random_{bernoulli,uniform,normal,log_normal}.cu): uniform draws in
+ * (lower, upper], Bernoulli as (u <= p) with u in (0, 1], normal and
+ * log-normal with (mean, sd).  The reference's GPU device takes its stream
+ * from cuRAND; here the stream is Philox4x32-10 (Salmon et al., SC'11),
+ * stateless: element i is word i%4 of the block with counter offset + i/4
+ * under the key `seed`.  The caller owns the position in the stream and moves
+ * `offset` on by (n + 3) / 4 after a call; a call with a smaller n yields a
+ * prefix of the same draw.  Normal draws use Box-Muller on word pairs. */
+int phip_random_uniform_f32(phip_ctx *ctx, uint64_t seed, uint64_t offset, float lower, float upper,
+                            float *y, size_t n);
+int phip_random_uniform_f16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float lower, float upper,
+                            void *y, size_t n);
+int phip_random_uniform_bf16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float lower, float upper,
+                            void *y, size_t n);
+int phip_random_bernoulli_f32(phip_ctx *ctx, uint64_t seed, uint64_t offset, float p, float *y, size_t n);
+int phip_random_bernoulli_f16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float p, void *y, size_t n);
+int phip_random_bernoulli_bf16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float p, void *y, size_t n);
+int phip_random_normal_f32(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                           float *y, size_t n);
+int phip_random_normal_f16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                           void *y, size_t n);
+int phip_random_normal_bf16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                           void *y, size_t n);
+int phip_random_log_normal_f32(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                               float *y, size_t n);
+int phip_random_log_normal_f16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                               void *y, size_t n);
+int phip_random_log_normal_bf16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
+                               void *y, size_t n);
+
 /* ---- timing ---------------------------------------------------------------
  * No counterpart in the reference (it has no profiling facility); events are
  * recorded on the context's stream so they bracket exactly the kernels the

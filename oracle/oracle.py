@@ -24,6 +24,7 @@ __all__ = [
     "batch_pick_bw", "batch_slice_fw", "batch_slice_bw", "batch_concat_fw", "transpose_fw",
     "transpose_bw", "permute_dims_fw", "permute_dims_bw", "flip_fw", "flip_bw", "reduce_fw",
     "extremum_bw", "arg_extremum", "broadcast_fw",
+    "RANDOM_KINDS", "philox4x32_10", "random",
 ]
 
 _F = ctypes.POINTER(ctypes.c_float)
@@ -103,6 +104,9 @@ def lib():
             getattr(l, name).argtypes = args
             getattr(l, name).restype = None
         l.ref_reduce_fw.argtypes = [_I, _F, _D, _U, _U, _U, _F]
+        l.ref_philox4x32_10.argtypes = [_D, _D, _D]
+        l.ref_philox4x32_10.restype = None
+        l.ref_random.argtypes = [_I, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float, _F, _Z]
         _lib = l
     return _lib
 
@@ -487,4 +491,24 @@ def broadcast_fw(x, dims, batch, dim, size):
     d, depth = _dims(dims)
     y = np.empty(x.size * size, dtype=np.float32)
     lib().ref_broadcast_fw(_p(x), d, depth, batch, dim, size, _p(y))
+    return y
+
+
+# ---- random tensors (ref_random.c) ---------------------------------------------
+RANDOM_KINDS = ["uniform", "bernoulli", "normal", "log_normal"]
+
+
+def philox4x32_10(counter, key):
+    """One Philox4x32-10 block: 4 counter words, 2 key words -> 4 output words."""
+    c = (_U * 4)(*[int(v) for v in counter])
+    k = (_U * 2)(*[int(v) for v in key])
+    out = (_U * 4)()
+    lib().ref_philox4x32_10(c, k, out)
+    return list(out)
+
+
+def random(kind, seed, offset, p0, p1, n):
+    """n draws: uniform (p0, p1], bernoulli(p0), normal / log_normal (mean p0, sd p1)."""
+    y = np.empty(n, dtype=np.float32)
+    _ok(lib().ref_random(RANDOM_KINDS.index(kind), seed, offset, p0, p1, _p(y), n), kind)
     return y

@@ -164,6 +164,18 @@ SIGNATURES = {
     "phip_reduce_fw_bf16": [_vp, _int, _vp, _vp, _u32, _u32, _u32],
     "phip_extremum_bw_bf16": [_vp, _int, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "phip_arg_extremum_bf16": [_vp, _int, _vp, _ids, _u32, _u32, _u32],
+    "phip_random_uniform_f32": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_bernoulli_f32": [_vp, _u64, _u64, _f, _vp, _sz],
+    "phip_random_normal_f32": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_log_normal_f32": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_uniform_f16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_bernoulli_f16": [_vp, _u64, _u64, _f, _vp, _sz],
+    "phip_random_normal_f16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_log_normal_f16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_uniform_bf16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_bernoulli_bf16": [_vp, _u64, _u64, _f, _vp, _sz],
+    "phip_random_normal_bf16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
+    "phip_random_log_normal_bf16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
     "phip_matmul_fw_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_f16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_bf16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],

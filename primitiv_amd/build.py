@@ -18,6 +18,7 @@ SOURCES = [
     "phip_pointwise_binary.hip",
     "phip_indexing.hip",
     "phip_reduce.hip",
+    "phip_random.hip",
     "phip_gemm_f32.hip",
     "phip_gemm_f32_direct.hip",
     "phip_gemm_f32_lds.hip",

@@ -8,6 +8,7 @@ the matmul path touches.  All arithmetic happens in libphip.so on the GPU; this
 file only checks shapes, owns handles and moves bytes.
 """
 import ctypes
+import os
 
 import numpy as np
 
@@ -354,7 +355,9 @@ class HIP:
         _lib.call("phip_ctx_create", int(device_id), ctypes.byref(self._ctx))
         self._ctx_id = _lib.lib().phip_ctx_id(self._ctx)
         self._device_id = int(device_id)
-        self._rng_seed = rng_seed
+        # devices/cuda/device.cc: without a seed the generator is seeded from std::random_device
+        self._rng_seed = int.from_bytes(os.urandom(8), "little") if rng_seed is None else int(rng_seed)
+        self._rng_offset = 0   # position in the Philox stream, in blocks of four draws
 
     def close(self):
         if self._ctx:
@@ -877,6 +880,39 @@ class HIP:
         _lib.call("phip_broadcast_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(), base, size,
                   x.shape().size() // base)
         return y
+
+    # -- random tensors ---------------------------------------------------------
+    def _random(self, kind, shape, *params):
+        y = self.new_raw_tensor(shape)
+        n = y.shape().size()
+        _lib.call("phip_random_%s_%s" % (kind, self._SUFFIX), self._ctx, self._rng_seed & (2 ** 64 - 1),
+                  self._rng_offset, *params, y.mutable_handle(), n)
+        self._rng_offset += (n + 3) // 4
+        return y
+
+    def random_bernoulli(self, shape, p):
+        # device.cc:107-114
+        if p < 0 or p > 1:
+            raise Error("Invalid Bernoulli probability: %g" % p)
+        return self._random("bernoulli", shape, float(p))
+
+    def random_uniform(self, shape, lower, upper):
+        # device.cc:116-126
+        if upper < lower:
+            raise Error("Invalid parameter of the uniform distribution. lower: %g, upper: %g" % (lower, upper))
+        return self._random("uniform", shape, float(lower), float(upper))
+
+    def random_normal(self, shape, mean, sd):
+        # device.cc:128-137
+        if sd <= 0:
+            raise Error("Invalid parameter of the normal distribution. mean: %g, SD: %g" % (mean, sd))
+        return self._random("normal", shape, float(mean), float(sd))
+
+    def random_log_normal(self, shape, mean, sd):
+        # device.cc:139-148
+        if sd <= 0:
+            raise Error("Invalid parameter of the log-normal distribution. mean: %g, SD: %g" % (mean, sd))
+        return self._random("log_normal", shape, float(mean), float(sd))
 
 
 class HIP16(HIP):

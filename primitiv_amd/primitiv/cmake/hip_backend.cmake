@@ -34,6 +34,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_pointwise_binary.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_indexing.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_reduce.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_random.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_direct.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip

@@ -206,7 +206,7 @@ bool HIP::check_support(std::uint32_t device_id) {
 }
 
 HIP::HIP(std::uint32_t device_id, std::uint32_t rng_seed, Storage storage)
-: dev_id_(device_id), rng_seed_(rng_seed), storage_(storage), ctx_(nullptr) {
+: dev_id_(device_id), rng_seed_(rng_seed), rng_offset_(0), storage_(storage), ctx_(nullptr) {
   assert_support(dev_id_);
   PHIP_CALL(::phip_ctx_create(static_cast<int>(dev_id_), &ctx_));
   phip_ctx *ctx = ctx_;
@@ -410,6 +410,29 @@ void HIP::inplace_subtract_impl(const Tensor &x, Tensor &y) {
 void HIP::inplace_multiply_const_impl(float k, Tensor &x) {
   PHIP_CALL(pointwise_abi(storage_).inplace_multiply_const(ctx_, k, get_mutable_handle(x), x.shape().size()));
 }
+
+// ---- random tensors ------------------------------------------------------------
+// Element i of a call is word i%4 of Philox block rng_offset_ + i/4; the
+// offset then moves past the blocks the call used.
+
+#define PHIP_DEF_RANDOM(name, ...) \
+  const std::size_t n = y.shape().size(); \
+  void *py = get_mutable_handle(y); \
+  switch (storage_) { \
+    case Storage::F32: \
+      PHIP_CALL(::phip_random_##name##_f32(ctx_, rng_seed_, rng_offset_, __VA_ARGS__, static_cast<float *>(py), n)); \
+      break; \
+    case Storage::F16: PHIP_CALL(::phip_random_##name##_f16(ctx_, rng_seed_, rng_offset_, __VA_ARGS__, py, n)); break; \
+    case Storage::BF16: PHIP_CALL(::phip_random_##name##_bf16(ctx_, rng_seed_, rng_offset_, __VA_ARGS__, py, n)); break; \
+  } \
+  rng_offset_ += (n + 3) / 4;
+
+void HIP::random_bernoulli_impl(float p, Tensor &y) { PHIP_DEF_RANDOM(bernoulli, p) }
+void HIP::random_uniform_impl(float lower, float upper, Tensor &y) { PHIP_DEF_RANDOM(uniform, lower, upper) }
+void HIP::random_normal_impl(float mean, float sd, Tensor &y) { PHIP_DEF_RANDOM(normal, mean, sd) }
+void HIP::random_log_normal_impl(float mean, float sd, Tensor &y) { PHIP_DEF_RANDOM(log_normal, mean, sd) }
+
+#undef PHIP_DEF_RANDOM
 
 // ---- moving and reducing along one dimension -------------------------------------
 // A tensor is seen around `dim` as [outer][n][base] (base = lower_volume(dim));

@@ -79,6 +79,12 @@ private:
   void inplace_subtract_impl(const Tensor &x, Tensor &y) override;
   void inplace_multiply_const_impl(float k, Tensor &x) override;
 
+  // random tensors: a Philox stream keyed by the seed; rng_offset_ is the position in it
+  void random_bernoulli_impl(float p, Tensor &y) override;
+  void random_uniform_impl(float lower, float upper, Tensor &y) override;
+  void random_normal_impl(float mean, float sd, Tensor &y) override;
+  void random_log_normal_impl(float mean, float sd, Tensor &y) override;
+
   // moving and reducing along one dimension
   std::vector<std::uint32_t> argmax_impl(const Tensor &x, std::uint32_t dim) override;
   std::vector<std::uint32_t> argmin_impl(const Tensor &x, std::uint32_t dim) override;
@@ -140,11 +146,7 @@ private:
   // ---- not implemented in this backend -------------------------------------
   [[noreturn]] static void unsupported(const char *op);
 
-#define PHIP_NI_RANDOM(name) \
-  void random_##name##_impl(float, float, Tensor &) override { unsupported("random_" #name); }
 
-  void random_bernoulli_impl(float, Tensor &) override { unsupported("random_bernoulli"); }
-  PHIP_NI_RANDOM(uniform) PHIP_NI_RANDOM(normal) PHIP_NI_RANDOM(log_normal)
 
   void conv2d_fw_impl(const Tensor &, const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t,
                       std::uint32_t, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("conv2d_fw"); }
@@ -157,7 +159,6 @@ private:
                           std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
                           Tensor &) override { unsupported("max_pool2d_bw"); }
 
-#undef PHIP_NI_RANDOM
 
   // Bytes of device storage for `n` elements (16-bit storage rounds the
   // element count up to even, as devices::CUDA16 does).
@@ -165,6 +166,7 @@ private:
 
   std::uint32_t dev_id_;
   std::uint32_t rng_seed_;
+  std::uint64_t rng_offset_;
   Storage storage_;
   // Declared before the pool so that it is destroyed after it: the pool's
   // deleter still needs the context while it frees its blocks.
