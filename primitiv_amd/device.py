@@ -452,12 +452,26 @@ class HIP:
         return self._download(x.handle(), x.shape().size())
 
     def copy_tensor(self, x):
-        # devices/cuda/ops/copy_tensor.cu:10-30: same storage type -> D2D,
-        # anything else bounces through the host.
+        # devices/cuda/ops/copy_tensor.cu:10-30.  Within one device the copy is
+        # ordered by the device's stream.  Between two devices on the same GPU
+        # (each has a stream of its own) the source is drained first and the
+        # copy, or the storage conversion, runs on the GPU; the destination is
+        # drained afterwards so that the source may be released at once.
+        # Anything else bounces through the host.
         ret = self.new_raw_tensor(x.shape())
-        if isinstance(x.device(), HIP) and x.device()._SUFFIX == self._SUFFIX:
-            _lib.call("phip_memcpy_d2d", self._ctx, ret._handle.ptr, x.handle(),
-                      self._elements_to_bytes(x.shape().size()))
+        src = x.device()
+        n = x.shape().size()
+        if src is self:
+            _lib.call("phip_memcpy_d2d", self._ctx, ret._handle.ptr, x.handle(), self._elements_to_bytes(n))
+        elif isinstance(src, HIP) and src._device_id == self._device_id and (
+                src._SUFFIX == self._SUFFIX or "f32" in (src._SUFFIX, self._SUFFIX)):
+            src.sync()
+            if src._SUFFIX == self._SUFFIX:
+                _lib.call("phip_memcpy_d2d", self._ctx, ret._handle.ptr, x.handle(), self._elements_to_bytes(n))
+            else:
+                _lib.call("phip_cvt_%s_to_%s" % (src._SUFFIX, self._SUFFIX), self._ctx, x.handle(),
+                          ret._handle.ptr, n)
+            self.sync()
         else:
             self.reset_tensor_by_array(x.to_vector(), ret)
         return ret

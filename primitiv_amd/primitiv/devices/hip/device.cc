@@ -313,15 +313,44 @@ void HIP::reset_tensor_by_array_impl(const float values[], Tensor &x) {
 
 void HIP::copy_tensor_impl(const Tensor &x, Tensor &y) {
   const DeviceType src = x.device().type();
+  const std::size_t n = x.shape().size();
   if (src == DeviceType::NAIVE || src == DeviceType::EIGEN) {
     // host tensors hand over their buffer directly
     reset_tensor_by_array(static_cast<const float *>(get_handle(x)), y);
-  } else if (src == type() && static_cast<const HIP &>(x.device()).storage_ == storage_) {
-    PHIP_CALL(::phip_memcpy_d2d(
-        ctx_, get_mutable_handle(y), get_handle(x), storage_bytes(x.shape().size())));
-  } else {
-    reset_tensor_by_vector(x.to_vector(), y);
+    return;
   }
+  if (src == DEVICE_TYPE_HIP || src == DEVICE_TYPE_HIP16) {
+    const HIP &from = static_cast<const HIP &>(x.device());
+    if (&from == this) {
+      // ordered by this device's stream
+      PHIP_CALL(::phip_memcpy_d2d(ctx_, get_mutable_handle(y), get_handle(x), storage_bytes(n)));
+      return;
+    }
+    const bool convertible = from.storage_ == storage_ || from.storage_ == Storage::F32 || storage_ == Storage::F32;
+    if (from.dev_id_ == dev_id_ && convertible) {
+      // Another device object on the same GPU has a stream of its own: drain
+      // it, copy or convert on the GPU, then drain this stream so that the
+      // source may be released as soon as the call returns.
+      PHIP_CALL(::phip_sync(from.ctx_));
+      void *py = get_mutable_handle(y);
+      const void *px = get_handle(x);
+      if (from.storage_ == storage_) {
+        PHIP_CALL(::phip_memcpy_d2d(ctx_, py, px, storage_bytes(n)));
+      } else if (from.storage_ == Storage::F16) {
+        PHIP_CALL(::phip_cvt_f16_to_f32(ctx_, px, static_cast<float *>(py), n));
+      } else if (from.storage_ == Storage::BF16) {
+        PHIP_CALL(::phip_cvt_bf16_to_f32(ctx_, px, static_cast<float *>(py), n));
+      } else if (storage_ == Storage::F16) {
+        PHIP_CALL(::phip_cvt_f32_to_f16(ctx_, static_cast<const float *>(px), py, n));
+      } else {
+        PHIP_CALL(::phip_cvt_f32_to_bf16(ctx_, static_cast<const float *>(px), py, n));
+      }
+      PHIP_CALL(::phip_sync(ctx_));
+      return;
+    }
+  }
+  // other devices, other GPUs, f16 <-> bf16: through the host
+  reset_tensor_by_vector(x.to_vector(), y);
 }
 
 void HIP::identity_impl(Tensor &y) {

@@ -118,6 +118,25 @@ def test_copy_between_devices(devs):
     other.close()
 
 
+def test_copy_between_devices_waits_for_the_source(devs):
+    # every device object has a stream of its own: a copy to another object must
+    # see the kernels still queued on the source, and the source may be dropped at once
+    src, other = devs[0], pa.HIP(0)
+    n = 1 << 22
+    x = src.new_tensor_by_constant([n], 1.0)
+    for _ in range(20):
+        x = src.const_fw("add_const", x, 1.0)
+    y = other.copy_tensor(x)
+    del x
+    assert np.array_equal(y.to_vector(), np.full(n, 21, np.float32))
+    for d16 in devs[1:]:
+        z = d16.copy_tensor(other.const_fw("add_const", y, 1.0))     # fp32 -> 16-bit on the GPU
+        assert np.array_equal(z.to_vector(), np.full(n, 22, np.float32))
+        back = other.copy_tensor(d16.const_fw("multiply_const", z, 2.0))   # and back
+        assert np.array_equal(back.to_vector(), np.full(n, 44, np.float32))
+    other.close()
+
+
 def test_inplace_add_golden(devs, golden):
     for d in devs:
         for c in golden["inplace_add"]:
