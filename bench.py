@@ -215,6 +215,40 @@ def measure_pointwise(reps=20):
                   % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
                   file=sys.stderr, flush=True)
         del x, y, g, g2, bias, gbias, xb, gxb, sbias, sx, sg, sgb, cases
+        # moving and reducing along a dimension: a 4096 x 4096 matrix with a minibatch of 4
+        # (64 Mi elements) and the softmax of a 10000-word vocabulary over a minibatch of 64
+        r, bs = 4096, 4
+        m = dev.new_tensor_by_constant(S([r, r], bs), 0.5)
+        gm = dev.new_tensor_by_constant(S([r, r], bs), 0.0)
+        whole = r * r * bs * item
+        logits = dev.new_tensor_by_constant(S([10000], 64), 0.5)
+        table = dev.new_tensor_by_constant(S([650, 10000]), 0.5)
+        gtable = dev.new_tensor_by_constant(S([650, 10000]), 0.0)
+        ids = [(7919 * i) % 10000 for i in range(64)]
+        picked = dev.pick_fw(table, ids, 1)
+        half = dev.slice_fw(m, 0, 0, r // 2)
+        cases = [
+            ("slice_fw_rows", lambda: dev.slice_fw(m, 0, 0, r // 2), whole),
+            ("slice_bw_rows", lambda: dev.slice_bw(half, 0, 0, gm), whole // 2 * 3),
+            ("concat_fw_cols", lambda: dev.concat_fw([half, half], 1), whole * 2),
+            ("transpose_fw", lambda: dev.transpose_fw(m), 2 * whole),
+            ("sum_fw_dim0", lambda: dev.reduce_fw("sum", m, 0), whole + whole // r),
+            ("sum_fw_dim1", lambda: dev.reduce_fw("sum", m, 1), whole + whole // r),
+            ("max_fw_dim1", lambda: dev.reduce_fw("max", m, 1), whole + whole // r),
+            ("logsumexp_fw_vocab", lambda: dev.reduce_fw("logsumexp", logits, 0), (640000 + 64) * item),
+            ("broadcast_fw_vocab", lambda: dev.broadcast_fw(dev.reduce_fw("sum", logits, 0), 0, 10000),
+             (2 * 640000 + 128) * item),
+            ("pick_fw_embedding", lambda: dev.pick_fw(table, ids, 1), 2 * 650 * 64 * item),
+            ("pick_bw_embedding", lambda: dev.pick_bw(picked, ids, 1, gtable), 3 * 650 * 64 * item),
+        ]
+        for name, fn, nbytes in cases:
+            sec = _event_seconds(dev, fn, reps)
+            out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
+                        "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
+            print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
+                  % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
+                  file=sys.stderr, flush=True)
+        del m, gm, logits, table, gtable, picked, half, cases
         dev.close()
     return out
 

@@ -108,21 +108,30 @@ __global__ __launch_bounds__(kBlock) void batch_pick_bw_kernel(const T *gy, cons
 
 // ---- transpose ------------------------------------------------------------------
 
-// 32 x 32 tiles through LDS: reads run along the source's columns, writes
-// along the destination's.  dst (cols x rows) (=|+=) transpose(src (rows x cols)).
+// 64 x 64 tiles through LDS: a wavefront reads 64 consecutive elements of a
+// source column and writes 64 consecutive elements of a destination column; the
+// 16 loads of a thread are all issued before the first LDS write.
+// dst (cols x rows) (=|+=) transpose(src (rows x cols)).
+constexpr uint32_t kTr = 64;
+
 template <typename T, bool ACC>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(const T *src, T *dst, uint32_t rows, uint32_t cols) {
-  __shared__ float tile[32][33];
+  __shared__ float tile[kTr][kTr + 1];
   const size_t ofs = (size_t)blockIdx.z * rows * cols;
-  const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  const uint32_t i0 = blockIdx.x * 32, j0 = blockIdx.y * 32;
-  for (uint32_t jj = ty; jj < 32; jj += 8) {
-    const uint32_t i = i0 + tx, j = j0 + jj;
-    if (i < rows && j < cols) tile[jj][tx] = to_f32(src[ofs + i + (size_t)j * rows]);
+  const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const uint32_t i0 = blockIdx.x * kTr, j0 = blockIdx.y * kTr;
+  float v[kTr / 4];
+#pragma unroll
+  for (uint32_t u = 0; u < kTr / 4; ++u) {
+    const uint32_t i = i0 + tx, j = j0 + ty + 4 * u;
+    v[u] = i < rows && j < cols ? to_f32(src[ofs + i + (size_t)j * rows]) : 0.f;
   }
+#pragma unroll
+  for (uint32_t u = 0; u < kTr / 4; ++u) tile[ty + 4 * u][tx] = v[u];
   __syncthreads();
-  for (uint32_t ii = ty; ii < 32; ii += 8) {
-    const uint32_t i = i0 + ii, j = j0 + tx;
+#pragma unroll
+  for (uint32_t u = 0; u < kTr / 4; ++u) {
+    const uint32_t ii = ty + 4 * u, i = i0 + ii, j = j0 + tx;
     if (i < rows && j < cols) put<T, ACC>(dst + ofs + j + (size_t)i * cols, tile[tx][ii]);
   }
 }
@@ -301,8 +310,8 @@ int transpose(phip_ctx *ctx, bool accumulate, const void *src, void *dst, uint32
   PHIP_ENTER(ctx);
   if (rows == 0 || cols == 0 || bs == 0) return PHIP_OK;
   PHIP_REQUIRE(src != nullptr && dst != nullptr, "null pointer");
-  PHIP_REQUIRE(bs <= 65535u && (cols + 31) / 32 <= 65535u, "shape exceeds what one launch covers");
-  const dim3 grid((rows + 31) / 32, (cols + 31) / 32, bs);
+  PHIP_REQUIRE(bs <= 65535u && (cols + kTr - 1) / kTr <= 65535u, "shape exceeds what one launch covers");
+  const dim3 grid((rows + kTr - 1) / kTr, (cols + kTr - 1) / kTr, bs);
   if (accumulate) {
     hipLaunchKernelGGL((transpose_kernel<T, true>), grid, dim3(kBlock), 0, ctx->stream, static_cast<const T *>(src),
                        static_cast<T *>(dst), rows, cols);

@@ -1,12 +1,21 @@
 // Reductions along one dimension of a tensor seen as [outer][n][base]:
 // sum, logsumexp, max, min, the gradient of max / min, and argmax / argmin.
 //
-// Two launch shapes.  "Column": one thread per output element walks the n
-// inputs in order; neighbouring threads read neighbouring addresses when
-// base > 1, and a thread reads a contiguous run when base == 1.  "Block":
-// one 256-thread workgroup per output element, for long reductions with few
-// outputs; the threads' partial results are combined through LDS by a tree of
-// fixed shape.  Either way a result does not depend on scheduling.
+// Four launch shapes, all built on one combiner interface (state, push, merge):
+//  * "rows"   (base == 1, n >= 32): a wavefront per output; its lanes stride
+//    along the contiguous n axis (256 bytes per load instruction), four
+//    independent partial states per lane keep four loads in flight, then the
+//    lanes combine by a butterfly of fixed shape.
+//  * "tiles"  (base >= 16): a workgroup is TX lanes along base (contiguous) by
+//    TY lanes that split n; four partial states per thread, then the TY
+//    partials combine through LDS in order.
+//  * "block"  (few outputs, long n): one 256-thread workgroup per output with
+//    an LDS tree of fixed shape.
+// When "tiles" or "block" would start too few workgroups to fill the chip, n is
+// cut into ranges reduced independently into partial states, which a second
+// small launch merges in order.
+//  * "column" (everything else, i.e. short reductions): one thread per output.
+// A result never depends on scheduling; no atomics are used.
 #include <vector>
 
 #include "phip_pointwise.h"
@@ -104,40 +113,202 @@ __global__ __launch_bounds__(kBlock) void reduce_column_kernel(const T *x, T *y,
   }
 }
 
-// One workgroup per output element; thread t takes j = t, t + 256, ...
+// Four independent partial states over j = first, first + step, ... < end: the
+// loads of four consecutive steps are in flight together; the partials merge in
+// a fixed order.
+template <typename T, typename OP>
+__device__ inline typename OP::State walk(const T *p, size_t stride_elems, uint32_t first, uint32_t step,
+                                          uint32_t end) {
+  typename OP::State st[4] = {OP::init(), OP::init(), OP::init(), OP::init()};
+  uint32_t j = first;
+  for (; j < end && end - j > 3 * step; j += 4 * step) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = to_f32(p[(size_t)(j + u * step) * stride_elems]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) OP::push(st[u], v[u], j + u * step);
+  }
+  for (int u = 0; j < end; j += step, ++u) OP::push(st[u & 3], to_f32(p[(size_t)j * stride_elems]), j);
+  OP::merge(st[0], st[1]);
+  OP::merge(st[2], st[3]);
+  OP::merge(st[0], st[2]);
+  return st[0];
+}
+
+// A long reduction may be cut into `splits` ranges of `chunk` positions, each
+// reduced by its own workgroup into partial[(o*splits + sp)*base + i]; a second
+// launch (reduce_finish_kernel) merges the ranges in order.  splits == 1 writes
+// the result directly.
+struct Split {
+  uint32_t splits, chunk;
+};
+
+template <typename T, typename OP, Emit EMIT>
+__device__ inline void finish(const typename OP::State &st, typename OP::State *partial, Split sp, uint32_t r,
+                              T *y, uint32_t *index_out, const T *gy, T *gx, size_t o, uint32_t i, uint32_t base,
+                              uint32_t n) {
+  if (sp.splits > 1) {
+    partial[(o * sp.splits + r) * base + i] = st;
+  } else {
+    emit<T, OP, EMIT>(st, y, index_out, gy, gx, o * base + i, o * n * base + i, base, n);
+  }
+}
+
+// One workgroup per (output element, range); thread t takes j = lo + t, lo + t + 256, ...
 template <typename T, typename OP, Emit EMIT>
 __global__ __launch_bounds__(kBlock) void reduce_block_kernel(const T *x, T *y, uint32_t *index_out, const T *gy,
-                                                               T *gx, uint32_t base, uint32_t n, size_t outputs) {
+                                                               T *gx, typename OP::State *partial, Split sp,
+                                                               uint32_t base, uint32_t n, size_t outputs) {
   __shared__ typename OP::State part[kBlock];
-  for (size_t q = blockIdx.x; q < outputs; q += gridDim.x) {
+  for (size_t b = blockIdx.x; b < outputs * sp.splits; b += gridDim.x) {
+    const size_t q = b / sp.splits;
+    const uint32_t r = (uint32_t)(b - q * sp.splits);
     const size_t o = q / base;
-    const size_t first = o * n * base + (q - o * base);
-    typename OP::State st = OP::init();
-    const T *p = x + first;
-    for (uint32_t j = threadIdx.x; j < n; j += kBlock) OP::push(st, to_f32(p[(size_t)j * base]), j);
-    part[threadIdx.x] = st;
+    const uint32_t i = (uint32_t)(q - o * base);
+    const uint32_t lo = r * sp.chunk, hi = n - lo < sp.chunk ? n : lo + sp.chunk;
+    part[threadIdx.x] = walk<T, OP>(x + o * n * base + i, base, lo + threadIdx.x, kBlock, hi);
     __syncthreads();
     for (int w = kBlock / 2; w > 0; w >>= 1) {
       if ((int)threadIdx.x < w) OP::merge(part[threadIdx.x], part[threadIdx.x + w]);
       __syncthreads();
     }
-    if (threadIdx.x == 0) emit<T, OP, EMIT>(part[0], y, index_out, gy, gx, q, first, base, n);
+    if (threadIdx.x == 0) finish<T, OP, EMIT>(part[0], partial, sp, r, y, index_out, gy, gx, o, i, base, n);
     __syncthreads();
   }
+}
+
+// base == 1: wavefront w of the grid owns outputs w, w + waves, ...; its lanes
+// stride along the contiguous run.
+template <typename T, typename OP, Emit EMIT>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const T *x, T *y, uint32_t *index_out, const T *gy,
+                                                              T *gx, uint32_t n, size_t outputs) {
+  const uint32_t lane = threadIdx.x & 63;
+  const size_t waves = (size_t)gridDim.x * (kBlock / 64);
+  for (size_t q = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); q < outputs; q += waves) {
+    const size_t first = q * n;
+    typename OP::State st = walk<T, OP>(x + first, 1, lane, 64, n);
+#pragma unroll
+    for (int w = 32; w > 0; w >>= 1) {
+      typename OP::State other;
+      unsigned char *dst = reinterpret_cast<unsigned char *>(&other);
+      const unsigned char *src = reinterpret_cast<const unsigned char *>(&st);
+#pragma unroll
+      for (unsigned k = 0; k < sizeof(st) / 4; ++k) {
+        int word;
+        __builtin_memcpy(&word, src + 4 * k, 4);
+        word = __shfl_down(word, w, 64);
+        __builtin_memcpy(dst + 4 * k, &word, 4);
+      }
+      if (lane < (uint32_t)w) OP::merge(st, other);
+    }
+    if (lane == 0) emit<T, OP, EMIT>(st, y, index_out, gy, gx, q, first, 1, n);
+  }
+}
+
+// base >= 16: threads (tx, ty); tx walks base (contiguous), ty splits the
+// range of n that the workgroup owns.
+template <typename T, typename OP, Emit EMIT, int TX>
+__global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, uint32_t *index_out, const T *gy,
+                                                               T *gx, typename OP::State *partial, Split sp,
+                                                               uint32_t base, uint32_t n, uint32_t outer) {
+  constexpr int TY = kBlock / TX;
+  __shared__ typename OP::State part[TY][TX];
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const uint32_t per_o = (base + TX - 1) / TX;
+  for (size_t b = blockIdx.x; b < (size_t)per_o * outer * sp.splits; b += gridDim.x) {
+    const uint32_t r = (uint32_t)(b % sp.splits);
+    const size_t t = b / sp.splits;
+    const size_t o = t / per_o;
+    const uint32_t i = (uint32_t)(t - o * per_o) * TX + tx;
+    const uint32_t lo = r * sp.chunk, hi = n - lo < sp.chunk ? n : lo + sp.chunk;
+    typename OP::State st = OP::init();
+    if (i < base) st = walk<T, OP>(x + o * n * base + i, base, lo + ty, TY, hi);
+    part[ty][tx] = st;
+    __syncthreads();
+    if (ty == 0 && i < base) {
+      for (int u = 1; u < TY; ++u) OP::merge(st, part[u][tx]);
+      finish<T, OP, EMIT>(st, partial, sp, r, y, index_out, gy, gx, o, i, base, n);
+    }
+    __syncthreads();
+  }
+}
+
+// Merges the ranges of one output in order: thread per output.
+template <typename T, typename OP, Emit EMIT>
+__global__ __launch_bounds__(kBlock) void reduce_finish_kernel(const typename OP::State *partial, uint32_t splits,
+                                                                T *y, uint32_t *index_out, const T *gy, T *gx,
+                                                                uint32_t base, uint32_t n, size_t outputs) {
+  for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < outputs; q += (size_t)gridDim.x * kBlock) {
+    const size_t o = q / base;
+    const uint32_t i = (uint32_t)(q - o * base);
+    typename OP::State st = partial[(o * splits) * base + i];
+    for (uint32_t r = 1; r < splits; ++r) OP::merge(st, partial[(o * splits + r) * base + i]);
+    emit<T, OP, EMIT>(st, y, index_out, gy, gx, q, o * n * base + i, base, n);
+  }
+}
+
+// How many ranges to cut n into so that `groups` workgroups become about four
+// per compute unit, each range at least `min_chunk` long.
+inline Split choose_split(size_t groups, uint32_t n, uint32_t min_chunk, size_t cus) {
+  Split sp = {1, n};
+  const size_t want = 4 * cus;
+  if (groups >= want || n < 2 * min_chunk) return sp;
+  size_t splits = (want + groups - 1) / groups;
+  const size_t most = n / min_chunk;
+  if (splits > most) splits = most;
+  if (splits < 2) return sp;
+  sp.chunk = (uint32_t)((n + splits - 1) / splits);
+  sp.splits = (uint32_t)((n + sp.chunk - 1) / sp.chunk);
+  return sp;
 }
 
 template <typename T, typename OP, Emit EMIT>
 int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T *gy, T *gx, uint32_t base,
                   uint32_t n, uint32_t outer) {
+  typedef typename OP::State State;
   const size_t outputs = (size_t)base * outer;
   const size_t cus = (size_t)ctx->prop.multiProcessorCount;
-  const bool by_block = n >= 64 && (base == 1 || outputs < 16 * cus) && outputs < 64 * cus;
+  const size_t cap = cus * 16;
+  const bool by_block = n >= 256 && outputs < 2 * cus;
+  const bool by_rows = !by_block && base == 1 && n >= 32;
+  const bool by_tiles = !by_block && !by_rows && base >= 16 && n >= 16;
+  if (!by_block && !by_tiles) {
+    if (by_rows) {
+      const size_t blocks = (outputs + kBlock / 64 - 1) / (kBlock / 64);
+      hipLaunchKernelGGL((reduce_rows_kernel<T, OP, EMIT>), dim3((unsigned)(blocks < cap ? blocks : cap)),
+                         dim3(kBlock), 0, ctx->stream, x, y, index_out, gy, gx, n, outputs);
+    } else {
+      hipLaunchKernelGGL((reduce_column_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
+                         ctx->stream, x, y, index_out, gy, gx, base, n, outputs);
+    }
+    PHIP_LAUNCH_CHECK();
+    return PHIP_OK;
+  }
+  const int tx = base >= 64 ? 64 : 16;
+  const size_t groups = by_block ? outputs : (size_t)((base + tx - 1) / tx) * outer;
+  const Split sp = choose_split(groups, n, by_block ? 16384 : 256, cus);
+  void *block = nullptr;
+  if (sp.splits > 1) {
+    const int rc = phip_pool_alloc(ctx, sizeof(State) * outputs * sp.splits, &block, nullptr);
+    if (rc != PHIP_OK) return rc;
+  }
+  State *partial = static_cast<State *>(block);
+  const size_t blocks = groups * sp.splits;
+  const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
   if (by_block) {
-    hipLaunchKernelGGL((reduce_block_kernel<T, OP, EMIT>), dim3((unsigned)outputs), dim3(kBlock), 0, ctx->stream, x,
-                       y, index_out, gy, gx, base, n, outputs);
+    hipLaunchKernelGGL((reduce_block_kernel<T, OP, EMIT>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out, gy,
+                       gx, partial, sp, base, n, outputs);
+  } else if (tx == 64) {
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
+                       gy, gx, partial, sp, base, n, outer);
   } else {
-    hipLaunchKernelGGL((reduce_column_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
-                       ctx->stream, x, y, index_out, gy, gx, base, n, outputs);
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 16>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
+                       gy, gx, partial, sp, base, n, outer);
+  }
+  if (sp.splits > 1) {
+    hipLaunchKernelGGL((reduce_finish_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
+                       ctx->stream, partial, sp.splits, y, index_out, gy, gx, base, n, outputs);
+    phip_pool_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
   }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;

@@ -181,6 +181,37 @@ def test_dimension_ops_match_oracle(dev, dims, batch):
     assert np.allclose(gx.to_vector(), oracle.permute_dims_bw(y.to_vector(), g0, dims, perm, batch), atol=1e-6)
 
 
+# One shape per launch shape of the reduction (wavefront per contiguous run, lanes
+# along base with n split, workgroup per output, thread per output), ragged sizes.
+REDUCE_SHAPES = [([100, 300], 2, 0), ([33, 1031], 1, 0), ([70, 100], 3, 1), ([129, 517], 2, 1), ([20, 50], 40, 1),
+                 ([17, 1000, 3], 1, 1), ([5000], 3, 0), ([20011], 2, 0), ([3, 9000], 2, 1), ([40, 20], 30, 0), ([4, 64, 2], 5, 1)]
+
+
+@pytest.mark.parametrize("dims,batch,dim", REDUCE_SHAPES)
+def test_reduction_launch_shapes_match_oracle(dev, dims, batch, dim):
+    rng = np.random.default_rng(dims[0] * 7 + batch)
+    n = int(np.prod(dims)) * batch
+    # few distinct values: ties everywhere, so the first-occurrence rule is exercised
+    for x in (rng.standard_normal(n).astype(np.float32), rng.integers(-3, 4, n).astype(np.float32)):
+        tx = dev.new_tensor_by_vector(S(dims, batch), x)
+        for op in pa.HIP.REDUCE_OPS:
+            got = dev.reduce_fw(op, tx, dim).to_vector()
+            want = oracle.reduce_fw(op, x, dims, batch, dim)
+            if op in ("max", "min"):
+                assert np.array_equal(got, want)
+            else:
+                assert np.allclose(got, want, rtol=1e-5, atol=2e-4)
+        for op in ("max", "min"):
+            assert np.array_equal(dev.arg_extremum(op, tx, dim), oracle.arg_extremum(op, x, dims, batch, dim))
+            yv = oracle.reduce_fw(op, x, dims, batch, dim)
+            gyv = rng.standard_normal(yv.size).astype(np.float32)
+            g0 = rng.standard_normal(n).astype(np.float32)
+            sy = tx.shape().resize_dim(dim, 1)
+            gx = dev.new_tensor_by_vector(S(dims, batch), g0)
+            dev.extremum_bw(op, tx, dev.new_tensor_by_vector(sy, yv), dev.new_tensor_by_vector(sy, gyv), dim, gx)
+            assert np.allclose(gx.to_vector(), oracle.extremum_bw(x, yv, gyv, g0, dims, batch, dim), atol=1e-6)
+
+
 @pytest.mark.parametrize("d1,d2,bs", [(1, 1, 1), (5, 7, 3), (64, 32, 2), (100, 257, 4), (1000, 33, 1)])
 def test_transpose_and_batch_ops_match_oracle(dev, d1, d2, bs):
     rng = np.random.default_rng(d1 + d2)
