@@ -71,21 +71,47 @@ __global__ __launch_bounds__(kBlock) void pick_fw_kernel(const T *x, const IdLis
   }
 }
 
-// gx[b*sx + ...] += gy[b][t]; with sx == 0 every sample lands in the same gx
-// and the thread that owns t walks the samples in order.
-template <typename T>
+// Longest index list for which a workgroup row per sample is started (each row
+// scans the list once).
+constexpr uint32_t kOwnerSamples = 1024;
+
+// Samples that pick the same index add into the same place of a shared gx.
+// The first sample b that picks an index owns it: it adds, in sample order, the
+// gradient of every sample that picks the same index; the others leave.  The
+// result is the sequential sum whatever the schedule, and distinct indices
+// proceed in parallel.  `b` is uniform over the workgroup.
+__device__ inline bool owns_index(const IdList &ids, uint32_t b, uint32_t si) {
+  const uint32_t id = ids[b * si];
+  for (uint32_t p = 0; p < b; ++p)
+    if (ids[p * si] == id) return false;
+  return true;
+}
+
+// gx[b*sx + ...] += gy[b][t].  sx != 0: every sample has its own gx.  sx == 0
+// and OWNERS: workgroup row b handles the samples that share ids[b] (see
+// owns_index).  sx == 0 otherwise (very long lists): the thread that owns t
+// walks the samples in order.
+template <typename T, bool OWNERS>
 __global__ __launch_bounds__(kBlock) void pick_bw_kernel(const T *gy, const IdList ids, T *gx, uint32_t base,
                                                           uint32_t n, uint32_t sy, size_t sx, uint32_t si,
                                                           uint32_t bs) {
+  const uint32_t b = blockIdx.y;
+  if (OWNERS && sx == 0 && !owns_index(ids, b, si)) return;
   for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < sy; t += gridDim.x * kBlock) {
     const uint32_t o = t / base, i = t - o * base;
     const size_t within = (size_t)o * base * n + i;
     if (sx != 0) {
-      const uint32_t b = blockIdx.y;
       put<T, true>(gx + b * sx + (size_t)ids[b * si] * base + within, to_f32(gy[(size_t)b * sy + t]));
-    } else if (blockIdx.y == 0) {
-      for (uint32_t b = 0; b < bs; ++b)
-        put<T, true>(gx + (size_t)ids[b * si] * base + within, to_f32(gy[(size_t)b * sy + t]));
+    } else if (OWNERS) {
+      const uint32_t id = ids[b * si];
+      T *g = gx + (size_t)id * base + within;
+      float acc = to_f32(*g);
+      for (uint32_t p = b; p < bs; ++p)
+        if (ids[p * si] == id) acc = to_f32(from_f32<T>(acc + to_f32(gy[(size_t)p * sy + t])));
+      *g = from_f32<T>(acc);
+    } else {
+      for (uint32_t p = 0; p < bs; ++p)
+        put<T, true>(gx + (size_t)ids[p * si] * base + within, to_f32(gy[(size_t)p * sy + t]));
     }
   }
 }
@@ -98,12 +124,26 @@ __global__ __launch_bounds__(kBlock) void batch_pick_fw_kernel(const T *x, const
     y[(size_t)b * sy + t] = px[t];
 }
 
-// gx[ids[b]][t] += gy[b][t]: indices may repeat, so the owner of t walks b in order.
-template <typename T>
+// gx[ids[b]][t] += gy[b][t]: indices may repeat.  OWNERS: workgroup row b handles
+// the samples that share ids[b] (see owns_index); otherwise the owner of t
+// walks b in order.
+template <typename T, bool OWNERS>
 __global__ __launch_bounds__(kBlock) void batch_pick_bw_kernel(const T *gy, const IdList ids, T *gx, uint32_t sy,
                                                                 uint32_t bs) {
-  for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < sy; t += gridDim.x * kBlock)
-    for (uint32_t b = 0; b < bs; ++b) put<T, true>(gx + (size_t)ids[b] * sy + t, to_f32(gy[(size_t)b * sy + t]));
+  const uint32_t b = blockIdx.y;
+  if (OWNERS && !owns_index(ids, b, 1)) return;
+  for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < sy; t += gridDim.x * kBlock) {
+    if (OWNERS) {
+      const uint32_t id = ids[b];
+      T *g = gx + (size_t)id * sy + t;
+      float acc = to_f32(*g);
+      for (uint32_t p = b; p < bs; ++p)
+        if (ids[p] == id) acc = to_f32(from_f32<T>(acc + to_f32(gy[(size_t)p * sy + t])));
+      *g = from_f32<T>(acc);
+    } else {
+      for (uint32_t p = 0; p < bs; ++p) put<T, true>(gx + (size_t)ids[p] * sy + t, to_f32(gy[(size_t)p * sy + t]));
+    }
+  }
 }
 
 // ---- transpose ------------------------------------------------------------------
@@ -273,8 +313,11 @@ int pick(phip_ctx *ctx, bool forward, const void *src, const uint32_t *ids, uint
   if (forward) {
     hipLaunchKernelGGL(pick_fw_kernel<T>, grid2(sy, bs, ctx), dim3(kBlock), 0, ctx->stream,
                        static_cast<const T *>(src), list.list, static_cast<T *>(dst), base, n, sy, sx, si);
+  } else if (sx != 0 || bs <= kOwnerSamples) {
+    hipLaunchKernelGGL((pick_bw_kernel<T, true>), grid2(sy, bs, ctx), dim3(kBlock), 0, ctx->stream,
+                       static_cast<const T *>(src), list.list, static_cast<T *>(dst), base, n, sy, sx, si, bs);
   } else {
-    hipLaunchKernelGGL(pick_bw_kernel<T>, grid2(sy, sx ? bs : 1, ctx), dim3(kBlock), 0, ctx->stream,
+    hipLaunchKernelGGL((pick_bw_kernel<T, false>), grid2(sy, 1, ctx), dim3(kBlock), 0, ctx->stream,
                        static_cast<const T *>(src), list.list, static_cast<T *>(dst), base, n, sy, sx, si, bs);
   }
   release_ids(ctx, &list);
@@ -295,8 +338,11 @@ int batch_pick(phip_ctx *ctx, bool forward, const void *src, const uint32_t *ids
   if (forward) {
     hipLaunchKernelGGL(batch_pick_fw_kernel<T>, grid2(volume, n_ids, ctx), dim3(kBlock), 0, ctx->stream,
                        static_cast<const T *>(src), list.list, static_cast<T *>(dst), volume);
+  } else if (n_ids <= kOwnerSamples) {
+    hipLaunchKernelGGL((batch_pick_bw_kernel<T, true>), grid2(volume, n_ids, ctx), dim3(kBlock), 0, ctx->stream,
+                       static_cast<const T *>(src), list.list, static_cast<T *>(dst), volume, n_ids);
   } else {
-    hipLaunchKernelGGL(batch_pick_bw_kernel<T>, dim3(blocks_for(volume, ctx)), dim3(kBlock), 0, ctx->stream,
+    hipLaunchKernelGGL((batch_pick_bw_kernel<T, false>), grid2(volume, 1, ctx), dim3(kBlock), 0, ctx->stream,
                        static_cast<const T *>(src), list.list, static_cast<T *>(dst), volume, n_ids);
   }
   release_ids(ctx, &list);

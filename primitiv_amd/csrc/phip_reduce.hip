@@ -113,25 +113,33 @@ __global__ __launch_bounds__(kBlock) void reduce_column_kernel(const T *x, T *y,
   }
 }
 
-// Four independent partial states over j = first, first + step, ... < end: the
-// loads of four consecutive steps are in flight together; the partials merge in
-// a fixed order.
-template <typename T, typename OP>
+// U independent partial states over j = first, first + step, ... < end: the
+// loads of U consecutive steps are in flight together; the partials merge in a
+// fixed order.
+template <typename T, typename OP, int U = 4>
 __device__ inline typename OP::State walk(const T *p, size_t stride_elems, uint32_t first, uint32_t step,
                                           uint32_t end) {
-  typename OP::State st[4] = {OP::init(), OP::init(), OP::init(), OP::init()};
+  typename OP::State st[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) st[u] = OP::init();
   uint32_t j = first;
-  for (; j < end && end - j > 3 * step; j += 4 * step) {
-    float v[4];
+  for (; j < end && end - j > (U - 1) * step; j += U * step) {
+    float v[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = to_f32(p[(size_t)(j + u * step) * stride_elems]);
+    for (int u = 0; u < U; ++u) v[u] = to_f32(p[(size_t)(j + u * step) * stride_elems]);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) OP::push(st[u], v[u], j + u * step);
+    for (int u = 0; u < U; ++u) OP::push(st[u], v[u], j + u * step);
   }
-  for (int u = 0; j < end; j += step, ++u) OP::push(st[u & 3], to_f32(p[(size_t)j * stride_elems]), j);
-  OP::merge(st[0], st[1]);
-  OP::merge(st[2], st[3]);
-  OP::merge(st[0], st[2]);
+#pragma unroll
+  for (int u = 0; u < U - 1; ++u) {
+    if (j < end) OP::push(st[u], to_f32(p[(size_t)j * stride_elems]), j);
+    j += step;
+  }
+#pragma unroll
+  for (int w = 1; w < U; w *= 2) {
+#pragma unroll
+    for (int u = 0; u + w < U; u += 2 * w) OP::merge(st[u], st[u + w]);
+  }
   return st[0];
 }
 
@@ -166,7 +174,7 @@ __global__ __launch_bounds__(kBlock) void reduce_block_kernel(const T *x, T *y, 
     const size_t o = q / base;
     const uint32_t i = (uint32_t)(q - o * base);
     const uint32_t lo = r * sp.chunk, hi = n - lo < sp.chunk ? n : lo + sp.chunk;
-    part[threadIdx.x] = walk<T, OP>(x + o * n * base + i, base, lo + threadIdx.x, kBlock, hi);
+    part[threadIdx.x] = walk<T, OP, 8>(x + o * n * base + i, base, lo + threadIdx.x, kBlock, hi);
     __syncthreads();
     for (int w = kBlock / 2; w > 0; w >>= 1) {
       if ((int)threadIdx.x < w) OP::merge(part[threadIdx.x], part[threadIdx.x + w]);
@@ -286,7 +294,7 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
   }
   const int tx = base >= 64 ? 64 : 16;
   const size_t groups = by_block ? outputs : (size_t)((base + tx - 1) / tx) * outer;
-  const Split sp = choose_split(groups, n, by_block ? 16384 : 256, cus);
+  const Split sp = choose_split(groups, n, by_block ? 8192 : 256, cus);
   void *block = nullptr;
   if (sp.splits > 1) {
     const int rc = phip_pool_alloc(ctx, sizeof(State) * outputs * sp.splits, &block, nullptr);

@@ -242,10 +242,12 @@ def test_transpose_and_batch_ops_match_oracle(dev, d1, d2, bs):
     assert np.array_equal(joined.to_vector(), oracle.batch_concat_fw([x, picked.to_vector(), x]))
 
 
-def test_long_index_lists_go_through_device_memory(dev):
-    # more indices than travel in the kernel arguments
+@pytest.mark.parametrize("bs", [700, 1500])
+def test_long_index_lists_go_through_device_memory(dev, bs):
+    # more indices than travel in the kernel arguments (700), and more than get a
+    # workgroup row each in the gradient (1500); many samples share an index
     rng = np.random.default_rng(5)
-    vocab, width, bs = 500, 48, 700
+    vocab, width = 500, 48
     table = rng.standard_normal(width * vocab).astype(np.float32)
     ids = [int(i) for i in rng.integers(0, vocab, bs)]
     t = dev.new_tensor_by_vector(S([width, vocab]), table)
@@ -254,8 +256,15 @@ def test_long_index_lists_go_through_device_memory(dev):
     assert np.array_equal(got.to_vector(), oracle.pick_fw(table, [width, vocab], 1, ids, 1))
     g = dev.new_tensor_by_constant(S([width, vocab]), 0)
     dev.pick_bw(got, ids, 1, g)
-    assert np.allclose(g.to_vector(), oracle.pick_bw(got.to_vector(), np.zeros_like(table), [width, vocab], 1, ids, 1),
-                       rtol=1e-5, atol=1e-5)
+    # fp32, samples added in order: the same sums as the sequential restatement
+    assert np.array_equal(g.to_vector(), oracle.pick_bw(got.to_vector(), np.zeros_like(table), [width, vocab], 1, ids, 1))
+    # the same lists through batch_pick: a table of `vocab` samples
+    tb = dev.new_tensor_by_vector(S([width], vocab), table)
+    gotb = dev.batch_pick_fw(tb, ids)
+    assert np.array_equal(gotb.to_vector(), got.to_vector())
+    gb = dev.new_tensor_by_constant(S([width], vocab), 0)
+    dev.batch_pick_bw(gotb, ids, gb)
+    assert np.array_equal(gb.to_vector(), g.to_vector())
 
 
 def test_softmax_cross_entropy_pieces(dev):
