@@ -34,6 +34,28 @@ __global__ __launch_bounds__(kBlock) void copy_rows_kernel(const T *src, T *dst,
   }
 }
 
+// The same copy in 16-byte packs: span, the strides and both addresses are
+// multiples of a pack, and every argument counts packs.
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kBlock) void copy_rows_pack_kernel(const T *src, T *dst, uint32_t span, uint32_t total,
+                                                                 size_t ss, size_t ds, uint32_t bs, size_t sbs,
+                                                                 size_t dbs) {
+  constexpr int N = Pack<T>::N;
+  for (uint32_t idx = blockIdx.x * kBlock + threadIdx.x; idx < total; idx += gridDim.x * kBlock) {
+    const uint32_t r = idx / span, i = idx - r * span;
+    for (uint32_t b = blockIdx.y; b < bs; b += gridDim.y) {
+      Pack<T> v = load_pack(src + (b * sbs + r * ss + i) * N);
+      T *d = dst + (b * dbs + r * ds + i) * N;
+      if constexpr (ACC) {
+        const Pack<T> old = load_pack(d);
+#pragma unroll
+        for (int k = 0; k < N; ++k) v.v[k] = from_f32<T>(to_f32(old.v[k]) + to_f32(v.v[k]));
+      }
+      store_pack(d, v);
+    }
+  }
+}
+
 // dst[r*ds + i] += sum over b of src[b*sbs + r*ss + i], added in order of b.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void copy_rows_sum_kernel(const T *src, T *dst, uint32_t span, uint32_t total,
@@ -243,9 +265,22 @@ int copy_rows(phip_ctx *ctx, const void *src, void *dst, uint32_t span, uint32_t
   const uint32_t total = span * rows;
   const T *s = static_cast<const T *>(src);
   T *d = static_cast<T *>(dst);
+  constexpr uint32_t N = Pack<T>::N;
+  const bool packs = aligned16(src) && aligned16(dst) && span % N == 0 && ss % N == 0 && ds % N == 0 &&
+                     sbs % N == 0 && dbs % N == 0;
   if (dbs == 0 && bs > 1) {
     hipLaunchKernelGGL(copy_rows_sum_kernel<T>, dim3(blocks_for(total, ctx)), dim3(kBlock), 0, ctx->stream, s, d,
                        span, total, (size_t)ss, (size_t)ds, bs, (size_t)sbs);
+  } else if (packs) {
+    if (accumulate) {
+      hipLaunchKernelGGL((copy_rows_pack_kernel<T, true>), grid2(total / N, bs, ctx), dim3(kBlock), 0, ctx->stream, s,
+                         d, span / N, total / N, (size_t)(ss / N), (size_t)(ds / N), bs, (size_t)(sbs / N),
+                         (size_t)(dbs / N));
+    } else {
+      hipLaunchKernelGGL((copy_rows_pack_kernel<T, false>), grid2(total / N, bs, ctx), dim3(kBlock), 0, ctx->stream, s,
+                         d, span / N, total / N, (size_t)(ss / N), (size_t)(ds / N), bs, (size_t)(sbs / N),
+                         (size_t)(dbs / N));
+    }
   } else if (accumulate) {
     hipLaunchKernelGGL((copy_rows_kernel<T, true>), grid2(total, bs, ctx), dim3(kBlock), 0, ctx->stream, s, d, span,
                        total, (size_t)ss, (size_t)ds, bs, (size_t)sbs, (size_t)dbs);

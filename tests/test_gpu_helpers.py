@@ -137,6 +137,36 @@ def test_copy_between_devices_waits_for_the_source(devs):
     other.close()
 
 
+def test_checkpoint_round_trip(devs, tmp_path):
+    # a parameter file written from one device loads into any other
+    # (test/parameter_test.cc:284-322 runs the same round trip on one device);
+    # the file holds float32, so a 16-bit device rounds once on load and
+    # its own values survive save + load unchanged
+    from primitiv_amd import parameter_file as pf
+    rng = np.random.default_rng(3)
+    value = rng.standard_normal(300 * 70).astype(np.float32)
+    m1 = rng.standard_normal(300 * 70).astype(np.float32)
+    path = str(tmp_path / "param.data")
+    for src in devs:
+        v = src.new_tensor_by_vector(pa.Shape([300, 70]), value)
+        stats = {"adam-m1": src.new_tensor_by_vector(pa.Shape([300, 70]), m1),
+                 "adam-m2": src.new_tensor_by_constant(pa.Shape([300, 70]), 0.25)}
+        pf.save(path, v, stats)
+        held = v.to_vector()
+        for dst in devs:
+            got, st = pf.load(path, dst)
+            assert got.device() is dst and got.shape() == v.shape() and sorted(st) == ["adam-m1", "adam-m2"]
+            if dst is src or dst is devs[0]:
+                assert np.array_equal(got.to_vector(), held)              # nothing is lost
+                assert np.array_equal(st["adam-m1"].to_vector(), stats["adam-m1"].to_vector())
+            else:
+                assert np.allclose(got.to_vector(), held, rtol=8e-3, atol=1e-6)   # one rounding to 16 bits
+            assert np.array_equal(st["adam-m2"].to_vector(), np.full(300 * 70, 0.25, np.float32))
+            # the loaded tensor is a working operand on its device
+            y = dst.matmul_fw(dst.transpose_fw(got), got)
+            assert y.shape() == pa.Shape([70, 70])
+
+
 def test_inplace_add_golden(devs, golden):
     for d in devs:
         for c in golden["inplace_add"]:

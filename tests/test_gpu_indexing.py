@@ -324,3 +324,38 @@ def test_half_storage_matches_oracle(dev16):
     assert np.array_equal(dev16.transpose_fw(tx).to_vector(), oracle.transpose_fw(xr, 40, 30, batch))
     assert np.array_equal(dev16.permute_dims_fw(tx, [1, 0]).to_vector(), oracle.permute_dims_fw(xr, dims, [1, 0], batch))
     assert np.array_equal(dev16.batch_pick_fw(tx, [2, 2, 0]).to_vector(), oracle.batch_pick_fw(xr, 1200, [2, 2, 0]))
+
+
+def _aligned_copies(dev, exact_sum):
+    # extents and offsets that are multiples of 16 bytes in every storage type: the
+    # copies then move whole 16-byte packs
+    rng = np.random.default_rng(21)
+    dims, batch = [64, 48], 3
+    n = 64 * 48 * batch
+    tx = dev.new_tensor_by_vector(S(dims, batch), rng.standard_normal(n).astype(np.float32))
+    xr = tx.to_vector()
+    for dim, lo, up in ((0, 16, 56), (1, 8, 40), (0, 0, 64)):
+        y = dev.slice_fw(tx, dim, lo, up)
+        assert np.array_equal(y.to_vector(), oracle.slice_fw(xr, dims, batch, dim, lo, up))
+        g0 = dev.new_tensor_by_vector(S(dims, batch), rng.standard_normal(n).astype(np.float32))
+        g0v, yv = g0.to_vector(), y.to_vector()
+        dev.slice_bw(y, dim, lo, g0)
+        want = oracle.slice_bw(yv, batch, up - lo, g0v, dims, batch, dim, lo)
+        if exact_sum:
+            assert np.array_equal(g0.to_vector(), want)
+        else:
+            assert np.max(np.abs(g0.to_vector() - want)) <= 2e-2 * np.max(np.abs(want))
+    for dim in (0, 1, 2):
+        got = dev.concat_fw([tx, tx], dim)
+        want, wd, wb = oracle.concat_fw([(xr, dims, batch), (xr, dims, batch)], dim)
+        assert got.shape() == S(wd, wb)
+        assert np.array_equal(got.to_vector(), want)
+    assert np.array_equal(dev.batch_slice_fw(tx, 1, 3).to_vector(), xr[64 * 48:])
+
+
+def test_aligned_copies_match_oracle(dev):
+    _aligned_copies(dev, True)
+
+
+def test_half_storage_aligned_copies_match_oracle(dev16):
+    _aligned_copies(dev16, False)
