@@ -22,6 +22,7 @@ SOURCES = [
     "phip_gemm_f32.hip",
     "phip_gemm_f32_direct.hip",
     "phip_gemm_f32_lds.hip",
+    "phip_gemm_f32_slab.hip",
     "phip_gemm_h16.hip",
     "phip_gemm_h16_big.hip",
     "phip_matmul.hip",

@@ -337,7 +337,9 @@ int launch_tile(phip_ctx *ctx, const Gemm &p, GemmArgs a, bool vec_a, bool vec_b
 int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return PHIP_OK;
   bool handled = false;
-  int rc = gemm_f32_direct(ctx, p, &handled);
+  int rc = gemm_f32_slab(ctx, p, &handled);
+  if (rc != PHIP_OK || handled) return rc;
+  rc = gemm_f32_direct(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;
   rc = gemm_f32_lds(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;

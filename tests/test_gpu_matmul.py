@@ -210,6 +210,40 @@ def test_large_tile_f32(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(gb, rgb) <= F32_TOL
 
 
+# a large operand streamed against at most 64 output columns (the output-projection
+# products): 32 x 64 tiles with the K range cut between workgroups.  Aligned and
+# 4-byte-aligned narrow operands, ragged M / N / K, N = 1, a contraction over
+# the minibatch, a minibatch of large operands.
+STREAMED_F32 = [  # di, dj, dk, ba, bb
+    (4100, 520, 1, 1, 64),
+    (4100, 518, 1, 1, 40),
+    (1028, 512, 48, 5, 1),
+    (8192, 260, 1, 1, 1),
+    (4100, 520, 2, 1, 30),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", STREAMED_F32)
+def test_streamed_operand_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di + dj + dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    y, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(y, ry) <= F32_TOL
+    assert norm_rel_err(ga, rga) <= F32_TOL
+    assert norm_rel_err(gb, rgb) <= F32_TOL
+    # the second call's y lands in pool memory that still holds the first call's
+    # results: an overwriting product must not add to them (a split product zero-fills first)
+    y2, _, _ = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    assert norm_rel_err(y2, ry) <= F32_TOL
+
+
 # shapes that reach the 256x256x64 large-tile kernel with ragged edges in every
 # dimension (multiples of 8, not of 256 / 64), in each batch case
 BIG_H16 = [  # di, dj, dk, ba, bb
