@@ -339,6 +339,8 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   bool handled = false;
   int rc = gemm_f32_slab(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;
+  rc = gemm_f32_rankk(ctx, p, &handled);
+  if (rc != PHIP_OK || handled) return rc;
   rc = gemm_f32_direct(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;
   rc = gemm_f32_lds(ctx, p, &handled);

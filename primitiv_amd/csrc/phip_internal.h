@@ -110,6 +110,7 @@ int gemm_f32(phip_ctx *ctx, const Gemm &g);
 int gemm_f32_direct(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_slab(phip_ctx *ctx, const Gemm &g, bool *handled);
+int gemm_f32_rankk(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_h16(phip_ctx *ctx, const Gemm &g, Elem elem);
 int gemm_h16_big(phip_ctx *ctx, const Gemm &g, Elem elem, bool *handled);
 

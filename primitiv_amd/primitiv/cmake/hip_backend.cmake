@@ -39,6 +39,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_direct.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_slab.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_rankk.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16_big.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_matmul.hip

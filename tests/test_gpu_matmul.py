@@ -220,6 +220,12 @@ STREAMED_F32 = [  # di, dj, dk, ba, bb
     (1028, 512, 48, 5, 1),
     (8192, 260, 1, 1, 1),
     (4100, 520, 2, 1, 30),
+    # weight gradients that are rank-K updates (K = minibatch <= 64) of a large matrix:
+    # 128 x 128 tiles in one round; aligned and 4-byte-aligned x, K = 64 / 40 / 20, a minibatch of updates
+    (4100, 1300, 1, 1, 64),
+    (4100, 1302, 1, 1, 40),
+    (4100, 1300, 1, 1, 20),
+    (1028, 1300, 30, 4, 4),
 ]
 
 
