@@ -5,10 +5,12 @@
 // No LDS staging and no barriers in the K loop: every wavefront loads its
 // matrix-instruction operands straight from global memory, already in the
 // instruction's register layout, and keeps many independent loads in flight.
-// The four wavefronts of a workgroup share one (32*TM) x (32*TN) output tile
-// and split its K range between them; their partial tiles are summed through
-// LDS once, at the end.  K can also be split between workgroups, whose tiles
-// are then added into C with fp32 atomics.
+// The WAVES (4 or 8) wavefronts of a workgroup share one (32*TM) x (32*TN)
+// output tile and split its K range between them; their partial tiles are
+// summed through LDS once, at the end.  More wavefronts shorten the chain of
+// dependent load rounds of a long K without the zero fill and atomics that a
+// split between workgroups costs an overwriting product.  K can also be split
+// between workgroups, whose tiles are then added into C with fp32 atomics.
 //
 // K is walked in chunks of 8.  v_mfma_f32_32x32x2_f32 takes, per lane, one A
 // and one B value for k slot (lane / 32); the four instructions of a chunk use
@@ -59,10 +61,10 @@ __device__ inline void zero_outside(float (&v)[4], unsigned mask) {
   for (int e = 0; e < 4; ++e) v[e] = ((mask >> e) & 1u) ? v[e] : 0.0f;
 }
 
-template <int TM, int TN, int U, bool A_KMAJOR, bool B_KMAJOR, int VA, int VB>
-__global__ __launch_bounds__(kThreads) void gemm_f32_direct_kernel(const DirectArgs d) {
+template <int TM, int TN, int U, bool A_KMAJOR, bool B_KMAJOR, int VA, int VB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_f32_direct_kernel(const DirectArgs d) {
   const GemmArgs &g = d.g;
-  __shared__ float red[4 * TM * TN * 16 * 64];
+  __shared__ float red[WAVES * TM * TN * 16 * 64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -75,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_direct_kernel(const DirectA
   const int z = t / g.splits;
   const int m0 = tile_m * 32 * TM, n0 = tile_n * 32 * TN;
 
-  // chunks [cb, ce) belong to this workgroup; wave w takes cb + w, cb + w + 4, ...
+  // chunks [cb, ce) belong to this workgroup; wave w takes cb + w, cb + w + WAVES, ...
   const int cb = (int)((long)split * d.total_chunks / g.splits);
   const int ce = (int)((long)(split + 1) * d.total_chunks / g.splits);
 
@@ -91,13 +93,13 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_direct_kernel(const DirectA
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  for (int c0 = cb + wave; c0 < ce; c0 += 4 * U) {
+  for (int c0 = cb + wave; c0 < ce; c0 += WAVES * U) {
     float av[U][TM][4], bv[U][TN][4];
     unsigned am[U][TM], bm[U][TN];
     // all loads of U chunks first ...
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c0 + 4 * u;
+      const int c = c0 + WAVES * u;
       const bool live = c < ce;
       const int cc = live ? c : cb;
       const int r = cc / d.chunks_per_r;
@@ -133,8 +135,8 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_direct_kernel(const DirectA
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[u][j][e], av[u][i][e], acc[i][j], 0, 0, 0);
   }
 
-  // Sum the four waves' tiles: every wave parks its registers in LDS, then
-  // wave w reduces and writes registers [4w, 4w+4) of each 32x32 block.
+  // Sum the waves' tiles: every wave parks its registers in LDS, then wave w
+  // reduces and writes its share of the 16 registers of each 32x32 block.
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -149,22 +151,23 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_direct_kernel(const DirectA
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      float vals[4];
-      int ns[4];
+      constexpr int kShare = 16 / WAVES;  // registers of the block that this wave reduces
+      float vals[kShare];
+      int ns[kShare];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int v = wave * 4 + q;
+      for (int q = 0; q < kShare; ++q) {
+        const int v = wave * kShare + q;
         float s = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) s += red[(((w * TM + i) * TN + j) * 16 + v) * 64 + lane];
+        for (int w = 0; w < WAVES; ++w) s += red[(((w * TM + i) * TN + j) * 16 + v) * 64 + lane];
         vals[q] = s;
         ns[q] = 8 * (v / 4) + (v % 4);
       }
-      emit_c<4>(Cz, g.ldc, m0 + i * 32, n0 + j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic, g.accumulate);
+      emit_c<kShare>(Cz, g.ldc, m0 + i * 32, n0 + j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic, g.accumulate);
     }
 }
 
-template <int TM, int TN, int U>
+template <int TM, int TN, int U, int WAVES>
 int launch_direct(phip_ctx *ctx, const Gemm &p, DirectArgs d, int splits, bool vec_a, bool vec_b) {
   GemmArgs &a = d.g;
   a.tiles_m = (p.M + 32 * TM - 1) / (32 * TM);
@@ -183,8 +186,8 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, DirectArgs d, int splits, bool v
     PHIP_LAUNCH_CHECK();
   }
 #define PHIP_DIRECT_V(AK, BKM, VVA, VVB)                                                                 \
-  hipLaunchKernelGGL((gemm_f32_direct_kernel<TM, TN, U, AK, BKM, VVA, VVB>), dim3((unsigned)grid),       \
-                     dim3(kThreads), 0, ctx->stream, d)
+  hipLaunchKernelGGL((gemm_f32_direct_kernel<TM, TN, U, AK, BKM, VVA, VVB, WAVES>), dim3((unsigned)grid), \
+                     dim3(64 * WAVES), 0, ctx->stream, d)
   // only a k-contiguous operand has a 16-byte form
   if (!p.a_kmajor && p.b_kmajor) {
     if (vec_b) PHIP_DIRECT_V(false, true, 1, 4); else PHIP_DIRECT_V(false, true, 1, 1);
@@ -257,15 +260,25 @@ int gemm_f32_direct(phip_ctx *ctx, const Gemm &p, bool *handled) {
   if (cap < 1) cap = 1;
   if (p.accumulate || t * 8 <= cus) splits = (int)(want < cap ? want : cap);
   if (splits < 1) splits = 1;
-  const long chunks_per_wave = d.total_chunks / (4L * splits);
+  // An overwriting product whose K fits one round of loads of 8 wavefronts (at
+  // most 8 chunks each) takes 8 wavefronts per workgroup.  (16 wavefronts for a
+  // longer K measured slower than the split with its zero fill: a 1024-thread
+  // workgroup leaves each lane 128 registers, too few for 8 chunks in flight.)
+  int waves = 4;
+  if (!p.accumulate && splits == 1 && d.total_chunks > 32 && d.total_chunks <= 64) waves = 8;
+  const long chunks_per_wave = d.total_chunks / ((long)waves * splits);
 
   *handled = true;
-  if (wide) {
-    if (chunks_per_wave > 4) return launch_direct<1, 2, 8>(ctx, p, d, splits, vec_a, vec_b);
-    return launch_direct<1, 2, 4>(ctx, p, d, splits, vec_a, vec_b);
+  if (waves == 8) {
+    if (wide) return launch_direct<1, 2, 8, 8>(ctx, p, d, splits, vec_a, vec_b);
+    return launch_direct<1, 1, 8, 8>(ctx, p, d, splits, vec_a, vec_b);
   }
-  if (chunks_per_wave > 4) return launch_direct<1, 1, 8>(ctx, p, d, splits, vec_a, vec_b);
-  return launch_direct<1, 1, 4>(ctx, p, d, splits, vec_a, vec_b);
+  if (wide) {
+    if (chunks_per_wave > 4) return launch_direct<1, 2, 8, 4>(ctx, p, d, splits, vec_a, vec_b);
+    return launch_direct<1, 2, 4, 4>(ctx, p, d, splits, vec_a, vec_b);
+  }
+  if (chunks_per_wave > 4) return launch_direct<1, 1, 8, 4>(ctx, p, d, splits, vec_a, vec_b);
+  return launch_direct<1, 1, 4, 4>(ctx, p, d, splits, vec_a, vec_b);
 }
 
 }  // namespace phip
