@@ -213,29 +213,79 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const T *x, T *y, u
   }
 }
 
-// base >= 16: threads (tx, ty); tx walks base (contiguous), ty splits the
-// range of n that the workgroup owns.
-template <typename T, typename OP, Emit EMIT, int TX>
+// V adjacent columns per lane, fetched as one V*sizeof(T)-byte access: U
+// independent partial states per column over j = first, first + step, ... < end.
+template <typename T, typename OP, int V, int U = 4>
+__device__ inline void walk_cols(const T *p, size_t stride_elems, uint32_t first, uint32_t step, uint32_t end,
+                                 typename OP::State (&out)[V]) {
+  struct alignas(V * sizeof(T)) Cols {
+    T c[V];
+  };
+  typename OP::State st[U][V];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int k = 0; k < V; ++k) st[u][k] = OP::init();
+  uint32_t j = first;
+  for (; j < end && end - j > (U - 1) * step; j += U * step) {
+    Cols v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const Cols *>(p + (size_t)(j + u * step) * stride_elems);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < V; ++k) OP::push(st[u][k], to_f32(v[u].c[k]), j + u * step);
+  }
+#pragma unroll
+  for (int u = 0; u < U - 1; ++u) {
+    if (j < end) {
+      const Cols v = *reinterpret_cast<const Cols *>(p + (size_t)j * stride_elems);
+#pragma unroll
+      for (int k = 0; k < V; ++k) OP::push(st[u][k], to_f32(v.c[k]), j);
+    }
+    j += step;
+  }
+#pragma unroll
+  for (int w = 1; w < U; w *= 2) {
+#pragma unroll
+    for (int u = 0; u + w < U; u += 2 * w)
+#pragma unroll
+      for (int k = 0; k < V; ++k) OP::merge(st[u][k], st[u + w][k]);
+  }
+#pragma unroll
+  for (int k = 0; k < V; ++k) out[k] = st[0][k];
+}
+
+// base >= 16: threads (tx, ty); tx walks base (contiguous, V columns per
+// lane), ty splits the range of n that the workgroup owns.  V > 1 needs base
+// to be a multiple of V and x aligned to V elements.
+template <typename T, typename OP, Emit EMIT, int TX, int V>
 __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, uint32_t *index_out, const T *gy,
                                                                T *gx, typename OP::State *partial, Split sp,
                                                                uint32_t base, uint32_t n, uint32_t outer) {
   constexpr int TY = kBlock / TX;
-  __shared__ typename OP::State part[TY][TX];
+  __shared__ typename OP::State part[TY][TX][V];
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-  const uint32_t per_o = (base + TX - 1) / TX;
+  const uint32_t per_o = (base + TX * V - 1) / (TX * V);
   for (size_t b = blockIdx.x; b < (size_t)per_o * outer * sp.splits; b += gridDim.x) {
     const uint32_t r = (uint32_t)(b % sp.splits);
     const size_t t = b / sp.splits;
     const size_t o = t / per_o;
-    const uint32_t i = (uint32_t)(t - o * per_o) * TX + tx;
+    const uint32_t i = ((uint32_t)(t - o * per_o) * TX + tx) * V;
     const uint32_t lo = r * sp.chunk, hi = n - lo < sp.chunk ? n : lo + sp.chunk;
-    typename OP::State st = OP::init();
-    if (i < base) st = walk<T, OP>(x + o * n * base + i, base, lo + ty, TY, hi);
-    part[ty][tx] = st;
+    typename OP::State st[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) st[k] = OP::init();
+    if (i < base) walk_cols<T, OP, V>(x + o * n * base + i, base, lo + ty, TY, hi, st);
+#pragma unroll
+    for (int k = 0; k < V; ++k) part[ty][tx][k] = st[k];
     __syncthreads();
     if (ty == 0 && i < base) {
-      for (int u = 1; u < TY; ++u) OP::merge(st, part[u][tx]);
-      finish<T, OP, EMIT>(st, partial, sp, r, y, index_out, gy, gx, o, i, base, n);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        for (int u = 1; u < TY; ++u) OP::merge(st[k], part[u][tx][k]);
+        finish<T, OP, EMIT>(st[k], partial, sp, r, y, index_out, gy, gx, o, i + k, base, n);
+      }
     }
     __syncthreads();
   }
@@ -292,8 +342,11 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
     PHIP_LAUNCH_CHECK();
     return PHIP_OK;
   }
+  // 16-bit storage: two columns per lane (4-byte accesses) when base and the address allow
+  constexpr int kCols = sizeof(T) == 2 ? 2 : 1;
+  const bool wide = kCols > 1 && base >= 128 && base % kCols == 0 && reinterpret_cast<uintptr_t>(x) % (kCols * sizeof(T)) == 0;
   const int tx = base >= 64 ? 64 : 16;
-  const size_t groups = by_block ? outputs : (size_t)((base + tx - 1) / tx) * outer;
+  const size_t groups = by_block ? outputs : (size_t)((base + tx * (wide ? kCols : 1) - 1) / (tx * (wide ? kCols : 1))) * outer;
   const Split sp = choose_split(groups, n, by_block ? 8192 : 256, cus);
   void *block = nullptr;
   if (sp.splits > 1) {
@@ -306,11 +359,14 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
   if (by_block) {
     hipLaunchKernelGGL((reduce_block_kernel<T, OP, EMIT>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out, gy,
                        gx, partial, sp, base, n, outputs);
+  } else if (wide) {
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64, kCols>), grid, dim3(kBlock), 0, ctx->stream, x, y,
+                       index_out, gy, gx, partial, sp, base, n, outer);
   } else if (tx == 64) {
-    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64, 1>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
                        gy, gx, partial, sp, base, n, outer);
   } else {
-    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 16>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 16, 1>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
                        gy, gx, partial, sp, base, n, outer);
   }
   if (sp.splits > 1) {

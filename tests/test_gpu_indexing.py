@@ -359,3 +359,22 @@ def test_aligned_copies_match_oracle(dev):
 
 def test_half_storage_aligned_copies_match_oracle(dev16):
     _aligned_copies(dev16, False)
+
+
+@pytest.mark.parametrize("dims,batch,dim", [([130, 517], 2, 1), ([256, 40, 3], 1, 1), ([129, 300], 1, 1), ([64, 1031], 3, 0)])
+def test_half_storage_reduction_launch_shapes(dev16, dims, batch, dim):
+    # 16-bit storage reduces two columns per lane when the stride below the reduced
+    # dimension is even and at least 128 (first two shapes); odd and short strides and
+    # a leading-dimension reduction take the other launch shapes
+    rng = np.random.default_rng(dims[0] + batch)
+    n = int(np.prod(dims)) * batch
+    for x in (rng.standard_normal(n).astype(np.float32), rng.integers(-3, 4, n).astype(np.float32)):
+        tx = dev16.new_tensor_by_vector(S(dims, batch), x)
+        xr = tx.to_vector()
+        for op in ("max", "min"):
+            assert np.array_equal(dev16.reduce_fw(op, tx, dim).to_vector(), oracle.reduce_fw(op, xr, dims, batch, dim))
+            assert np.array_equal(dev16.arg_extremum(op, tx, dim), oracle.arg_extremum(op, xr, dims, batch, dim))
+        for op in ("sum", "logsumexp"):
+            want = oracle.reduce_fw(op, xr, dims, batch, dim)
+            got = dev16.reduce_fw(op, tx, dim).to_vector()
+            assert np.max(np.abs(got - want)) <= 2e-2 * np.max(np.abs(want))
