@@ -41,10 +41,11 @@ __device__ inline uint32_t frag_base(int group, int lane) {
   else return (uint32_t)((8 * group + 4 * half) * (ROWS * 4) + xl * 4);
 }
 
-// Read r of the kFragReads<KMAJOR> that fetch one 32-row block's fragments.
+// LDS reads that fetch the fragments of one 32-row block.
 template <bool KMAJOR>
 constexpr int kFragReads = KMAJOR ? 1 : 4;
 
+// Read r of them.
 template <bool KMAJOR, int ROWS>
 __device__ inline void frag_read(const unsigned char *region, uint32_t base, int block, int r, float (&v)[4]) {
   if constexpr (KMAJOR) {
