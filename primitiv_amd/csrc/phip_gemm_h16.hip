@@ -7,7 +7,10 @@
 // 16-byte accesses, one that is contiguous along m or n is transposed while it
 // is written to LDS.  Results are rounded to the storage type once, after the
 // whole K range has been accumulated in fp32; `C += ...` reads C, adds in fp32
-// and rounds once.
+// and rounds once.  When a long K meets few output tiles, the K range is cut
+// between workgroups that leave fp32 partial tiles in scratch memory, and a
+// second launch adds them in order, so the one rounding (and a result that
+// does not depend on scheduling) is kept.
 #include "phip_internal.h"
 #include "phip_types.h"
 
@@ -34,6 +37,8 @@ struct GemmArgsH {
   int ktiles_per_r;
   int total_ktiles;
   int accumulate;
+  int splits;       // workgroups that share one C tile, each taking a K range
+  float *partial;   // splits > 1: fp32 tiles, element (m, n) of (sample z, range s) at ((z*splits + s)*N + n)*M + m
 };
 
 __device__ inline int xcd_remap(int bid, int total) {
@@ -189,7 +194,8 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
   int t = xcd_remap(blockIdx.x, gridDim.x);
   const int tile_m = t % g.tiles_m; t /= g.tiles_m;
   const int tile_n = t % g.tiles_n; t /= g.tiles_n;
-  const int z = t;
+  const int split = t % g.splits;
+  const int z = t / g.splits;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const uint16_t *Az = g.A + (long)z * g.sA;
@@ -213,16 +219,18 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
     lb.load(Bz + (long)r * g.rB, g.ldb, n0, g.N, k0, g.K, tid);
   };
 
-  const int kt_end = g.total_ktiles;
-  if (kt_end > 0) {
-    fetch(0);
+  // K tiles [kt_begin, kt_end) belong to this workgroup
+  const int kt_begin = (int)((long)split * g.total_ktiles / g.splits);
+  const int kt_end = (int)((long)(split + 1) * g.total_ktiles / g.splits);
+  if (kt_end > kt_begin) {
+    fetch(kt_begin);
     la.store(lds, tid);
     lb.store(lds + 2 * kStageA, tid);
   }
   __syncthreads();
 
-  for (int kt = 0; kt < kt_end; ++kt) {
-    const int stage = kt & 1;
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int stage = (kt - kt_begin) & 1;
     const bool more = kt + 1 < kt_end;
     if (more) fetch(kt + 1);
 
@@ -251,6 +259,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
   }
 
   uint16_t *Cz = g.C + (long)z * g.sC;
+  float *Pz = g.partial + ((long)z * g.splits + split) * g.M * g.N;
   const int cm = m0 + wm * WTM + (lane & 31);
   const int cn = n0 + wn * WTN + 4 * (lane >> 5);
 
@@ -280,8 +289,12 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
           const int m = cm + i * 32;
           const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
           if (m < g.M && n < g.N) {
-            uint16_t *p = Cz + m + (long)n * g.ldc;
-            *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+            if (g.splits > 1) {
+              Pz[m + (long)n * g.M] = s;
+            } else {
+              uint16_t *p = Cz + m + (long)n * g.ldc;
+              *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+            }
           }
         }
   } else {
@@ -294,22 +307,66 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
           const int m = cm + i * 32;
           const int n = cn + j * 32 + 8 * (v / 4) + (v % 4);
           if (m < g.M && n < g.N) {
-            uint16_t *p = Cz + m + (long)n * g.ldc;
             const float s = acc[i][j][v];
-            *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+            if (g.splits > 1) {
+              Pz[m + (long)n * g.M] = s;
+            } else {
+              uint16_t *p = Cz + m + (long)n * g.ldc;
+              *p = round_c<BF16>(g.accumulate ? load_c<BF16>(p) + s : s);
+            }
           }
         }
   }
 }
 
+// C (=|+=) the sum, in order, of the `splits` fp32 partial tiles of every element; one rounding.
+template <bool BF16>
+__global__ __launch_bounds__(kThreads) void finish_split_h16_kernel(const float *partial, uint16_t *C, int M, int N,
+                                                                    long ldc, long sC, int batch, int splits,
+                                                                    int accumulate) {
+  const long per = (long)M * N;
+  const long total = per * batch;
+  for (long idx = (long)blockIdx.x * kThreads + threadIdx.x; idx < total; idx += (long)gridDim.x * kThreads) {
+    const long z = idx / per, e = idx - z * per;
+    const float *p = partial + z * splits * per + e;
+    float s = p[0];
+    for (int r = 1; r < splits; ++r) s += p[r * per];
+    uint16_t *c = C + z * sC + (e % M) + (e / M) * ldc;
+    *c = round_c<BF16>(accumulate ? load_c<BF16>(c) + s : s);
+  }
+}
+
 template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool BF16>
-int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8) {
+int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8, bool may_split = false) {
   a.tiles_m = (p.M + BM - 1) / BM;
   a.tiles_n = (p.N + BN - 1) / BN;
   a.ktiles_per_r = (p.K + BK - 1) / BK;
   a.total_ktiles = a.ktiles_per_r * p.rbatch;
-  const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
-  if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
+  const long tiles = (long)a.tiles_m * a.tiles_n * p.batch;
+  // Few tiles over a long K (the second launch has to pay for itself: at least 32 K tiles): cut K so
+  // that about two workgroups per compute unit run (never more workgroups than places, at least
+  // eight K tiles each, at most 64 MiB of partial tiles).
+  long splits = 1;
+  if (may_split && tiles > 0 && a.total_ktiles >= 32) {
+    splits = 2L * ctx->prop.multiProcessorCount / tiles;
+    if (splits > a.total_ktiles / 8) splits = a.total_ktiles / 8;
+    const long per_split = 4L * p.M * p.N * p.batch;
+    if (per_split > 0 && splits > (64L << 20) / per_split) splits = (64L << 20) / per_split;
+    if (splits < 1) splits = 1;
+  }
+  a.splits = (int)splits;
+  a.partial = nullptr;
+  void *block = nullptr;
+  if (splits > 1) {
+    const int rc = phip_pool_alloc(ctx, (size_t)(4L * p.M * p.N * p.batch * splits), &block, nullptr);
+    if (rc != PHIP_OK) return rc;
+    a.partial = static_cast<float *>(block);
+  }
+  const long grid = tiles * splits;
+  if (grid > 0x7fffffffL) {
+    if (block) phip_pool_free(ctx, block);
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
+  }
 
 #define PHIP_LAUNCH(AK, BKM, VV)                                                                          \
   hipLaunchKernelGGL((gemm_h16_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VV, BF16>), dim3((unsigned)grid), \
@@ -321,9 +378,19 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8) {
   } else if (p.a_kmajor && p.b_kmajor) {
     if (vec8) PHIP_LAUNCH(true, true, 8); else PHIP_LAUNCH(true, true, 1);
   } else {
+    if (block) phip_pool_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
 #undef PHIP_LAUNCH
+  if (splits > 1) {
+    const long total = (long)p.M * p.N * p.batch;
+    long blocks = (total + kThreads - 1) / kThreads;
+    const long cap = 8L * ctx->prop.multiProcessorCount;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((finish_split_h16_kernel<BF16>), dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream,
+                       a.partial, a.C, p.M, p.N, p.ldc, p.sC, p.batch, (int)splits, a.accumulate);
+    phip_pool_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
+  }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
 }
@@ -351,7 +418,7 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
   };
   if (tiles(128, 128) >= cus) return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
   if (tiles(64, 64) >= cus) return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
-  return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec8);
+  return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec8, true);
 }
 
 }  // namespace

@@ -290,6 +290,32 @@ def test_large_tile_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
         assert norm_rel_err(got, ref) <= ulp
 
 
+# few output tiles over a long K on the 16-bit devices: the K range is cut between
+# workgroups that leave fp32 partial tiles, summed in order by a second launch
+# (gb of the first two shapes, the forward product of the third)
+@pytest.mark.parametrize("which", ["f16", "bf16"])
+@pytest.mark.parametrize("di,dj,dk,ba,bb", [(4100, 520, 1, 1, 64), (2050, 130, 3, 1, 9), (70, 3000, 40, 1, 1),
+                                            (1030, 48, 24, 6, 1)])
+def test_long_k_few_tiles_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
+    d = dev16 if which == "f16" else devbf16
+    rng = np.random.default_rng(di + dj + dk + ba)
+    bs = max(ba, bb)
+    r16 = (lambda x: x.astype(np.float16).astype(np.float32)) if which == "f16" else \
+        (lambda x: (x.view(np.uint32) & 0xFFFF0000).view(np.float32))
+    # inputs exactly representable in 16 bits: only the output rounding is left
+    a = r16(rng.standard_normal(di * dj * ba).astype(np.float32))
+    b = r16(rng.standard_normal(dj * dk * bb).astype(np.float32))
+    gy = r16(rng.standard_normal(di * dk * bs).astype(np.float32))
+    ga0 = r16(rng.standard_normal(a.size).astype(np.float32))
+    gb0 = r16(rng.standard_normal(b.size).astype(np.float32))
+    y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    ulp = 2.0 ** -10 if which == "f16" else 2.0 ** -7
+    for got, ref in ((y, ry), (ga, rga), (gb, rgb)):
+        assert norm_rel_err(got, ref) <= ulp
+
+
 def test_f16_matches_oracle_on_rounded_inputs(dev16):
     # With inputs already representable in fp16 the only error left is the
     # final rounding of the output (<= 2^-11 relative per element) on top of
