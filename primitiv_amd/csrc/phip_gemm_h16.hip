@@ -169,7 +169,7 @@ __device__ inline uint16_t round_c(float x) {
   }
 }
 
-template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool A_KMAJOR, bool B_KMAJOR, int V, bool BF16>
+template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool A_KMAJOR, bool B_KMAJOR, int VA, int VB, bool BF16>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
   static_assert(WGM * WGN * WGK == 4, "four wavefronts per workgroup");
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -201,8 +201,8 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
   const uint16_t *Az = g.A + (long)z * g.sA;
   const uint16_t *Bz = g.B + (long)z * g.sB;
 
-  typename LoaderSelectH<A_KMAJOR, BM, BK, V>::type la;
-  typename LoaderSelectH<B_KMAJOR, BN, BK, V>::type lb;
+  typename LoaderSelectH<A_KMAJOR, BM, BK, VA>::type la;
+  typename LoaderSelectH<B_KMAJOR, BN, BK, VB>::type lb;
 
   float16v acc[TM][TN];
 #pragma unroll
@@ -337,7 +337,7 @@ __global__ __launch_bounds__(kThreads) void finish_split_h16_kernel(const float 
 }
 
 template <int BM, int BN, int BK, int WGM, int WGN, int WGK, bool BF16>
-int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8, bool may_split = false) {
+int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec_a, bool vec_b, bool may_split = false) {
   a.tiles_m = (p.M + BM - 1) / BM;
   a.tiles_n = (p.N + BN - 1) / BN;
   a.ktiles_per_r = (p.K + BK - 1) / BK;
@@ -368,19 +368,27 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec8, bool may
     return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
   }
 
-#define PHIP_LAUNCH(AK, BKM, VV)                                                                          \
-  hipLaunchKernelGGL((gemm_h16_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VV, BF16>), dim3((unsigned)grid), \
+#define PHIP_LAUNCH_V(AK, BKM, VVA, VVB)                                                                          \
+  hipLaunchKernelGGL((gemm_h16_kernel<BM, BN, BK, WGM, WGN, WGK, AK, BKM, VVA, VVB, BF16>), dim3((unsigned)grid),  \
                      dim3(kThreads), 0, ctx->stream, a)
+#define PHIP_LAUNCH(AK, BKM)                                                                                     \
+  do {                                                                                                           \
+    if (vec_a && vec_b) PHIP_LAUNCH_V(AK, BKM, 8, 8);                                                            \
+    else if (vec_a) PHIP_LAUNCH_V(AK, BKM, 8, 1);                                                                \
+    else if (vec_b) PHIP_LAUNCH_V(AK, BKM, 1, 8);                                                                \
+    else PHIP_LAUNCH_V(AK, BKM, 1, 1);                                                                           \
+  } while (0)
   if (!p.a_kmajor && p.b_kmajor) {
-    if (vec8) PHIP_LAUNCH(false, true, 8); else PHIP_LAUNCH(false, true, 1);
+    PHIP_LAUNCH(false, true);
   } else if (!p.a_kmajor && !p.b_kmajor) {
-    if (vec8) PHIP_LAUNCH(false, false, 8); else PHIP_LAUNCH(false, false, 1);
+    PHIP_LAUNCH(false, false);
   } else if (p.a_kmajor && p.b_kmajor) {
-    if (vec8) PHIP_LAUNCH(true, true, 8); else PHIP_LAUNCH(true, true, 1);
+    PHIP_LAUNCH(true, true);
   } else {
     if (block) phip_pool_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
+#undef PHIP_LAUNCH_V
 #undef PHIP_LAUNCH
   if (splits > 1) {
     const long total = (long)p.M * p.N * p.batch;
@@ -410,15 +418,16 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
   auto aligned = [](const void *ptr, long ld, long s, long r) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 8 == 0 && s % 8 == 0 && r % 8 == 0;
   };
-  const bool vec8 = aligned(p.A, p.lda, p.sA, p.rA) && aligned(p.B, p.ldb, p.sB, p.rB);
+  // 16-byte loads per operand: aligned rows (the loaders check the ragged edge per vector)
+  const bool vec_a = aligned(p.A, p.lda, p.sA, p.rA), vec_b = aligned(p.B, p.ldb, p.sB, p.rB);
 
   const int cus = ctx->prop.multiProcessorCount;
   auto tiles = [&](int bm, int bn) {
     return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch;
   };
-  if (tiles(128, 128) >= cus) return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
-  if (tiles(64, 64) >= cus) return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec8);
-  return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec8, true);
+  if (tiles(128, 128) >= cus) return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
+  if (tiles(64, 64) >= cus) return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
+  return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec_a, vec_b, true);
 }
 
 }  // namespace
