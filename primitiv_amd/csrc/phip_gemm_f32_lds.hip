@@ -173,9 +173,9 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
     if (rc != PHIP_OK) return rc;                                                               \
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), kLdsBytes, ctx->stream, d); \
   } while (0)
-  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(0, false, true);
-  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(1, false, false);
-  else PHIP_LDS(2, true, true);
+  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true);
+  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false);
+  else PHIP_LDS(kSlotGemmF32Lds + 2, true, true);
 #undef PHIP_LDS
   PHIP_LAUNCH_CHECK();
   *handled = true;

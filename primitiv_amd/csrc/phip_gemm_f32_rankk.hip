@@ -226,8 +226,8 @@ int gemm_f32_rankk(phip_ctx *ctx, const Gemm &p, bool *handled) {
     if (rc != PHIP_OK) return rc;                                                                     \
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), kRankLdsBytes, ctx->stream, d);   \
   } while (0)
-  if (vec_b) PHIP_RANKK(21, 4);
-  else PHIP_RANKK(22, 2);
+  if (vec_b) PHIP_RANKK(kSlotGemmF32RankK + 0, 4);
+  else PHIP_RANKK(kSlotGemmF32RankK + 1, 2);
 #undef PHIP_RANKK
   PHIP_LAUNCH_CHECK();
   *handled = true;

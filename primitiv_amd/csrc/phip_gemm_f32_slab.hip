@@ -278,13 +278,13 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kSlabLdsBytes, ctx->stream, d);  \
   } while (0)
   if (!p.a_kmajor && p.b_kmajor) {
-    if (vec_b) PHIP_SLAB_G(16, false, true, 4);
-    else PHIP_SLAB_G(17, false, true, 1);
+    if (vec_b) PHIP_SLAB_G(kSlotGemmF32Slab + 0, false, true, 4);
+    else PHIP_SLAB_G(kSlotGemmF32Slab + 1, false, true, 1);
   } else if (!p.a_kmajor && !p.b_kmajor) {
-    PHIP_SLAB_G(18, false, false, 4);
+    PHIP_SLAB_G(kSlotGemmF32Slab + 2, false, false, 4);
   } else {
-    if (vec_b) PHIP_SLAB_G(19, true, true, 4);
-    else PHIP_SLAB_G(20, true, true, 1);
+    if (vec_b) PHIP_SLAB_G(kSlotGemmF32Slab + 3, true, true, 4);
+    else PHIP_SLAB_G(kSlotGemmF32Slab + 4, true, true, 1);
   }
 #undef PHIP_SLAB_G
   PHIP_LAUNCH_CHECK();

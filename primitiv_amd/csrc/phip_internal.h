@@ -71,6 +71,15 @@ struct phip_event {
 
 namespace phip {
 
+// Bits of phip_ctx::lds_limit_raised: first slot of each kernel family that
+// asks for a dynamic LDS size (one slot per instantiation, counted from here).
+enum LdsSlot {
+  kSlotGemmF32Lds = 0,    // 3 instantiations
+  kSlotGemmH16Big = 8,    // 6
+  kSlotGemmF32Slab = 16,  // 5
+  kSlotGemmF32RankK = 21, // 2
+};
+
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on
 // the context's device; done once per context and kernel (`slot` < 32).
 inline int raise_lds_limit(phip_ctx *ctx, int slot, const void *kernel, int bytes) {
