@@ -388,7 +388,7 @@ int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
 #define PHIP_LDS(SLOT, AK, BKM)                                                                  \
   do {                                                                                           \
     auto kern = gemm_h16_lds_kernel<AK, BKM, BF16>;                                              \
-    const int rc = raise_lds_limit(ctx, kSlotGemmH16Big + (SLOT) + (BF16 ? 3 : 0),                             \
+    const int rc = raise_lds_limit(ctx, kSlotGemmH16Big + (SLOT) + (BF16 ? 3 : 0),               \
                                    reinterpret_cast<const void *>(kern), kLds2Bytes);            \
     if (rc != PHIP_OK) return rc;                                                                \
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLds2Bytes, ctx->stream, a);  \
