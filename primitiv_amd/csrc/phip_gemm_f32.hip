@@ -354,6 +354,8 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
   a.rA = p.rA; a.rB = p.rB;
   a.accumulate = p.accumulate ? 1 : 0;
+  a.partial = nullptr;
+  a.tickets = nullptr;
   a.atomic = 0;
 
   auto aligned = [](const void *ptr, long ld, long s, long r) {

@@ -27,8 +27,11 @@ struct GemmArgs {
   int splits;        // workgroups that share one C tile, each taking a K range
   int ktiles_per_r;  // ceil(K / BK)
   int total_ktiles;  // rbatch * ktiles_per_r
-  int atomic;        // 1: add the tile into C with atomics (split K)
-  int accumulate;    // 1: C += tile, 0: C = tile (ignored when atomic)
+  int atomic;        // split K: 1: add the tile into C with atomics; 2: leave an fp32 partial tile, the
+                     // last workgroup of the output tile to finish sums the partial tiles in order
+  int accumulate;    // 1: C += tile, 0: C = tile (ignored when atomic == 1)
+  float *partial;    // atomic == 2: element (m, n) of (sample z, range s) at ((z*splits + s)*N + n)*M + m
+  uint32_t *tickets; // atomic == 2: one zeroed counter per output tile, left zeroed
 };
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
@@ -99,6 +102,81 @@ __device__ inline void emit_c(float *Cz, long ldc, int row0, int col0, int lane,
         if (ok[q]) *p[q] = accumulate ? old[q] + vals[c + q] : vals[c + q];
     }
   }
+}
+
+// Split K without atomics on C and without a zero fill (GemmArgs::atomic == 2).
+// Every workgroup of an output tile stores its NV results per lane (positions
+// as for emit_c) into its range's partial tile and takes a ticket; the one
+// that draws the last ticket adds the ranges in order, for the same positions,
+// into `vals` and returns true: it then writes C.  Workgroups of one tile run
+// on different XCDs, each with an L2 of its own, so the partial tiles are
+// written and read with device-scope accesses (past the L2s) instead of being
+// published by fences, which would write back a whole L2 per workgroup (38 us
+// instead of 8 on a 256 x 128 product).  A workgroup's own stores have been
+// acknowledged (s_waitcnt) before it takes its ticket, and the ticket is a
+// device-scope atomic, so whoever draws the last one finds every partial tile.
+template <int NV>
+__device__ inline void store_partial(const GemmArgs &g, int z, int split, int row0, int col0, int lane,
+                                     const int (&nq)[NV], const float (&vals)[NV]) {
+  float *P = g.partial + ((long)z * g.splits + split) * g.M * g.N;
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+#pragma unroll
+  for (int q = 0; q < NV; ++q) {
+    const int n = ncol + nq[q];
+    if (m < g.M && n < g.N)
+      __hip_atomic_store(P + m + (long)n * g.M, vals[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int NV>
+__device__ inline void sum_partials(const GemmArgs &g, int z, int row0, int col0, int lane, const int (&nq)[NV],
+                                    float (&vals)[NV]) {
+  const float *P = g.partial + (long)z * g.splits * g.M * g.N;
+  const long per = (long)g.M * g.N;
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+  const float *p[NV];
+  bool ok[NV];
+#pragma unroll
+  for (int q = 0; q < NV; ++q) {
+    const int n = ncol + nq[q];
+    ok[q] = m < g.M && n < g.N;
+    p[q] = ok[q] ? P + m + (long)n * g.M : P;
+    vals[q] = 0.0f;
+  }
+  // eight ranges at a time: the loads of a batch are all in flight before the first is added
+  for (int r0 = 0; r0 < g.splits; r0 += 8) {
+    float part[8][NV];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int q = 0; q < NV; ++q)
+        part[u][q] = __hip_atomic_load(p[q] + (r0 + u < g.splits ? r0 + u : r0) * per, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int q = 0; q < NV; ++q)
+        if (r0 + u < g.splits) vals[q] += part[u][q];
+  }
+#pragma unroll
+  for (int q = 0; q < NV; ++q) vals[q] = ok[q] ? vals[q] : 0.0f;
+}
+
+// Called by all threads of the workgroup after their store_partial calls.
+__device__ inline bool last_of_tile(const GemmArgs &g, int tile_id, uint32_t *flag) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own partial results have arrived, before the ticket
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t ticket = __hip_atomic_fetch_add(g.tickets + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = ticket == (uint32_t)g.splits - 1u;
+    // nobody else touches this counter any more in this launch: leave it zeroed for the next one
+    if (last) __hip_atomic_store(g.tickets + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last ? 1u : 0u;
+  }
+  __syncthreads();
+  return *flag != 0;
 }
 
 __attribute__((unused)) __global__ __launch_bounds__(kThreads) void zero_c_kernel(float *C, int M, int N, long ldc, long sC, int batch) {

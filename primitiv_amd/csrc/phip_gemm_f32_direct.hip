@@ -147,22 +147,52 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_f32_direct_kernel(const Direc
 
   float *Cz = g.C + (long)z * g.sC;
   const bool interior = m0 + 32 * TM <= g.M && n0 + 32 * TN <= g.N;
+  constexpr int kShare = 16 / WAVES;  // registers of each block that this wave reduces
+  // this wave's share of block (i, j), summed over the waves: values and their column offsets
+  auto reduced = [&](int i, int j, float (&vals)[kShare], int (&ns)[kShare]) {
+#pragma unroll
+    for (int q = 0; q < kShare; ++q) {
+      const int v = wave * kShare + q;
+      float s = 0.0f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) s += red[(((w * TM + i) * TN + j) * 16 + v) * 64 + lane];
+      vals[q] = s;
+      ns[q] = 8 * (v / 4) + (v % 4);
+    }
+  };
+  if (g.atomic == 2) {
+    // K is split between workgroups: leave the partial tile; the last one of the tile adds them up
+    __shared__ uint32_t last_flag;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        float vals[kShare];
+        int ns[kShare];
+        reduced(i, j, vals, ns);
+        store_partial<kShare>(g, z, split, m0 + i * 32, n0 + j * 32, lane, ns, vals);
+      }
+    if (!last_of_tile(g, (z * g.tiles_n + tile_n) * g.tiles_m + tile_m, &last_flag)) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        float vals[kShare];
+        int ns[kShare];
+#pragma unroll
+        for (int q = 0; q < kShare; ++q) ns[q] = 8 * ((wave * kShare + q) / 4) + ((wave * kShare + q) % 4);
+        sum_partials<kShare>(g, z, m0 + i * 32, n0 + j * 32, lane, ns, vals);
+        emit_c<kShare>(Cz, g.ldc, m0 + i * 32, n0 + j * 32, lane, g.M, g.N, interior, ns, vals, 0, g.accumulate);
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      constexpr int kShare = 16 / WAVES;  // registers of the block that this wave reduces
       float vals[kShare];
       int ns[kShare];
-#pragma unroll
-      for (int q = 0; q < kShare; ++q) {
-        const int v = wave * kShare + q;
-        float s = 0.0f;
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) s += red[(((w * TM + i) * TN + j) * 16 + v) * 64 + lane];
-        vals[q] = s;
-        ns[q] = 8 * (v / 4) + (v % 4);
-      }
+      reduced(i, j, vals, ns);
       emit_c<kShare>(Cz, g.ldc, m0 + i * 32, n0 + j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic, g.accumulate);
     }
 }
@@ -174,16 +204,29 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, DirectArgs d, int splits, bool v
   a.tiles_n = (p.N + 32 * TN - 1) / (32 * TN);
   a.splits = splits;
   a.atomic = splits > 1;
+  a.partial = nullptr;
+  a.tickets = ctx->tile_tickets;
   const long grid = (long)a.tiles_m * a.tiles_n * p.batch * splits;
   if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
+  // An overwriting product that is split leaves fp32 partial tiles in scratch memory and lets the last
+  // workgroup of each tile add them (no zero fill of C, no atomics on it, one launch); the atomics
+  // remain for an accumulating product and as the fallback.
+  void *block = nullptr;
   if (a.atomic && !p.accumulate) {
-    const int cus = ctx->prop.multiProcessorCount;
-    const long total = (long)p.M * p.N * p.batch;
-    long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-    if (blocks > cus * 8L) blocks = cus * 8L;
-    hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N,
-                       p.ldc, p.sC, p.batch);
-    PHIP_LAUNCH_CHECK();
+    const long tiles = (long)a.tiles_m * a.tiles_n * p.batch;
+    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
+    if (tiles <= kTicketSlots && bytes <= (size_t)(64L << 20) && phip_pool_alloc(ctx, bytes, &block, nullptr) == PHIP_OK) {
+      a.atomic = 2;
+      a.partial = static_cast<float *>(block);
+    } else {
+      const int cus = ctx->prop.multiProcessorCount;
+      const long total = (long)p.M * p.N * p.batch;
+      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+      if (blocks > cus * 8L) blocks = cus * 8L;
+      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N,
+                         p.ldc, p.sC, p.batch);
+      PHIP_LAUNCH_CHECK();
+    }
   }
 #define PHIP_DIRECT_V(AK, BKM, VVA, VVB)                                                                 \
   hipLaunchKernelGGL((gemm_f32_direct_kernel<TM, TN, U, AK, BKM, VVA, VVB, WAVES>), dim3((unsigned)grid), \
@@ -199,9 +242,11 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, DirectArgs d, int splits, bool v
     else if (vec_b) PHIP_DIRECT_V(true, true, 1, 4);
     else PHIP_DIRECT_V(true, true, 1, 1);
   } else {
+    if (block) phip_pool_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
 #undef PHIP_DIRECT_V
+  if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
 }
@@ -252,8 +297,8 @@ int gemm_f32_direct(phip_ctx *ctx, const Gemm &p, bool *handled) {
   // Split K between workgroups until about two workgroups per CU are busy,
   // keeping at least 4 chunks (32 k) per wavefront (measured best on the
   // recurrent-gate and output-projection gradients).  An overwriting product
-  // is only split when it would otherwise leave most of the chip idle: the
-  // split needs a zero fill of C in front of it.
+  // is only split when it would otherwise leave most of the chip idle: its
+  // ranges meet through partial tiles in scratch memory.
   int splits = 1;
   const long want = (2L * cus + t - 1) / t;
   long cap = d.total_chunks / 16;

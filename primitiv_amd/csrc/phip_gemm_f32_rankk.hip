@@ -216,6 +216,8 @@ int gemm_f32_rankk(phip_ctx *ctx, const Gemm &p, bool *handled) {
   a.total_ktiles = a.ktiles_per_r;
   a.atomic = 0;
   a.accumulate = p.accumulate ? 1 : 0;
+  a.partial = nullptr;
+  a.tickets = nullptr;
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
 

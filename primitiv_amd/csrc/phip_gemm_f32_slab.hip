@@ -258,6 +258,8 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   a.total_ktiles = (int)total_ktiles;
   a.atomic = splits > 1;
   a.accumulate = p.accumulate ? 1 : 0;
+  a.partial = nullptr;
+  a.tickets = nullptr;
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
 

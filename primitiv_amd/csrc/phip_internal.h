@@ -37,6 +37,9 @@ struct phip_ctx {
   // Kernels whose dynamic-LDS limit has been raised on this context's device
   // (one bit per kernel, see phip::raise_lds_limit).
   uint32_t lds_limit_raised = 0;
+  // One counter per output tile of a launch whose workgroups share tiles (see
+  // phip::kTicketSlots); all zero between launches.
+  uint32_t *tile_tickets = nullptr;
 };
 
 struct phip_event {
@@ -70,6 +73,9 @@ struct phip_event {
 #define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
 
 namespace phip {
+
+// Entries of phip_ctx::tile_tickets.
+constexpr int kTicketSlots = 65536;
 
 // Bits of phip_ctx::lds_limit_raised: first slot of each kernel family that
 // asks for a dynamic LDS size (one slot per instantiation, counted from here).

@@ -107,7 +107,11 @@ int phip_ctx_create(int device_id, phip_ctx **out) {
   ctx->device = device_id;
   hipError_t e = hipGetDeviceProperties(&ctx->prop, device_id);
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->tile_tickets), sizeof(uint32_t) * phip::kTicketSlots);
+  if (e == hipSuccess) e = hipMemset(ctx->tile_tickets, 0, sizeof(uint32_t) * phip::kTicketSlots);
   if (e != hipSuccess) {
+    if (ctx->tile_tickets) (void)hipFree(ctx->tile_tickets);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return fail(PHIP_ERR_RUNTIME, "context creation failed: %s", hipGetErrorString(e));
   }
@@ -141,6 +145,7 @@ int phip_ctx_destroy(phip_ctx *ctx) {
     int r2 = phip::release_reserved_locked(ctx);
     if (r2 != PHIP_OK) rc = r2;
   }
+  if (ctx->tile_tickets && hipFree(ctx->tile_tickets) != hipSuccess) rc = fail(PHIP_ERR_RUNTIME, "hipFree failed");
   if (hipStreamDestroy(ctx->stream) != hipSuccess) {
     rc = fail(PHIP_ERR_RUNTIME, "hipStreamDestroy failed");
   }

@@ -250,6 +250,23 @@ def test_streamed_operand_f32(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(y2, ry) <= F32_TOL
 
 
+# an overwriting product with few output tiles and a long K is cut between workgroups
+# that meet through partial tiles, summed in a fixed order by whichever finishes last:
+# right, and the same bits on every run
+@pytest.mark.parametrize("di,dj,dk,ba,bb", [(256, 784, 1, 1, 128), (64, 3000, 1, 1, 40), (100, 5000, 33, 1, 1),
+                                            (48, 2048, 8, 3, 3)])
+def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di + dj)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    ta = dev.new_tensor_by_vector(pa.Shape([di, dj], ba), a)
+    tb = dev.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    first = dev.matmul_fw(ta, tb).to_vector()
+    assert norm_rel_err(first, oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)) <= F32_TOL
+    for _ in range(25):
+        assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), first)
+
+
 # shapes that reach the 256x256x64 large-tile kernel with ragged edges in every
 # dimension (multiples of 8, not of 256 / 64), in each batch case
 BIG_H16 = [  # di, dj, dk, ba, bb
