@@ -195,10 +195,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_slab_kernel(const LdsArg
 
   float *Cz = g.C + (long)z * g.sC;
   const bool interior = m0 + TBM <= g.M && TBN <= g.N;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    float vals[4];
-    int ns[4];
+  // this wave's share of block j, summed over the waves: values and their column offsets
+  auto reduced = [&](int j, float (&vals)[4], int (&ns)[4]) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int v = wave * 4 + q;
@@ -208,6 +206,34 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_slab_kernel(const LdsArg
       vals[q] = sum;
       ns[q] = 8 * (v / 4) + (v % 4);
     }
+  };
+  if (g.atomic == 2) {
+    // K is split between workgroups: leave the partial tile; the last one of the tile adds them up
+    __shared__ uint32_t last_flag;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float vals[4];
+      int ns[4];
+      reduced(j, vals, ns);
+      store_partial<4>(g, z, split, m0, j * 32, lane, ns, vals);
+    }
+    if (!last_of_tile(g, z * g.tiles_m + tile_m, &last_flag)) return;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float vals[4];
+      int ns[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ns[q] = 8 * ((wave * 4 + q) / 4) + ((wave * 4 + q) % 4);
+      sum_partials<4>(g, z, m0, j * 32, lane, ns, vals);
+      emit_c<4>(Cz, g.ldc, m0, j * 32, lane, g.M, g.N, interior, ns, vals, 0, g.accumulate);
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    float vals[4];
+    int ns[4];
+    reduced(j, vals, ns);
     emit_c<4>(Cz, g.ldc, m0, j * 32, lane, g.M, g.N, interior, ns, vals, g.atomic, g.accumulate);
   }
 }
@@ -237,7 +263,7 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   const int cus = ctx->prop.multiProcessorCount;
   if (a_bytes * p.rbatch * p.batch < (8L << 20) || total_ktiles > 0x7fffffffL || tiles > 0x3fffffffL) return PHIP_OK;
   // two workgroups fit a compute unit: fill those places at most once (a workgroup that has to wait for
-  // a place doubles the launch's duration), at least four stages each
+  // a place doubles the launch's duration), at least eight stages each
   long splits = 2L * cus / tiles;
   if (splits > total_ktiles / 8) splits = total_ktiles / 8;
   if (splits < 1) splits = 1;
@@ -263,13 +289,24 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
 
+  // An overwriting product that is split leaves fp32 partial tiles in scratch memory and lets the last
+  // workgroup of each tile add them; the atomics remain for an accumulating product and as the fallback
+  // (then behind a zero fill of C).
+  void *block = nullptr;
   if (a.atomic && !p.accumulate) {
-    const long total = (long)p.M * p.N * p.batch;
-    long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-    if (blocks > cus * 8L) blocks = cus * 8L;
-    hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N, p.ldc,
-                       p.sC, p.batch);
-    PHIP_LAUNCH_CHECK();
+    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
+    if (tiles <= kTicketSlots && bytes <= (size_t)(64L << 20) && phip_pool_alloc(ctx, bytes, &block, nullptr) == PHIP_OK) {
+      a.atomic = 2;
+      a.partial = static_cast<float *>(block);
+      a.tickets = ctx->tile_tickets;
+    } else {
+      const long total = (long)p.M * p.N * p.batch;
+      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+      if (blocks > cus * 8L) blocks = cus * 8L;
+      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N, p.ldc,
+                         p.sC, p.batch);
+      PHIP_LAUNCH_CHECK();
+    }
   }
   const long grid = tiles * splits;
 #define PHIP_SLAB_G(SLOT, AK, BKM, VB)                                                              \
@@ -289,6 +326,7 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
     else PHIP_SLAB_G(kSlotGemmF32Slab + 4, true, true, 1);
   }
 #undef PHIP_SLAB_G
+  if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
   PHIP_LAUNCH_CHECK();
   *handled = true;
   return PHIP_OK;
