@@ -37,6 +37,7 @@ struct GemmArgsH {
   int ktiles_per_r;
   int total_ktiles;
   int accumulate;
+  int vec_c;        // C is 16-byte aligned with M and ldc multiples of 8: 16-byte C accesses
   int splits;       // workgroups that share one C tile, each taking a K range
   float *partial;   // splits > 1: fp32 tiles, element (m, n) of (sample z, range s) at ((z*splits + s)*N + n)*M + m
 };
@@ -180,7 +181,11 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
   constexpr int kStageA = BM * S, kStageB = BN * S;
   constexpr int kTileBytes = 2 * (kStageA + kStageB) * 2;
   constexpr int kReduceBytes = WGK > 1 ? 4 * TM * TN * 16 * 64 * 4 : 0;
-  constexpr int kLdsBytes = kTileBytes > kReduceBytes ? kTileBytes : kReduceBytes;
+  // write-out through LDS: per wavefront one 32-column block of its tile in fp32, [column][row]
+  constexpr int kColPitch = WTM + 8;  // floats; the pad staggers the columns over the banks
+  constexpr int kEmitBytes = WGK == 1 ? 4 * 32 * kColPitch * 4 : 0;
+  constexpr int kLdsMax1 = kTileBytes > kReduceBytes ? kTileBytes : kReduceBytes;
+  constexpr int kLdsBytes = kLdsMax1 > kEmitBytes ? kLdsMax1 : kEmitBytes;
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLdsBytes];
   uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
 
@@ -297,6 +302,46 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(const GemmArgsH g) {
             }
           }
         }
+  } else if (g.vec_c && g.splits == 1) {
+    // The matrix instruction leaves a lane with one row and 16 columns of each 32 x 32 block; C wants
+    // 8 consecutive rows of a column per lane (16 bytes).  Each 32-column block of the wave's tile is
+    // turned through an LDS area of the wave's own: written the way the accumulators lie, read back 8
+    // rows at a time.  M is a multiple of 8: a lane's 8 rows are inside or outside together.
+    float *area = reinterpret_cast<float *>(lds_raw) + wave * 32 * kColPitch;
+    constexpr int kLanesPerCol = WTM / 8;           // 4 or 8 lanes cover a column of the tile
+    constexpr int kColsPerPass = 64 / kLanesPerCol;
+    const int r0 = 8 * (lane % kLanesPerCol), c_in_pass = lane / kLanesPerCol;
+    const int m = m0 + wm * WTM + r0;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          area[(8 * (v / 4) + 4 * (lane >> 5) + (v % 4)) * kColPitch + 32 * i + (lane & 31)] = acc[i][j][v];
+      // the area belongs to this wave alone: its own LDS accesses stay in order
+#pragma unroll
+      for (int pass = 0; pass < 32 / kColsPerPass; ++pass) {
+        const int c = pass * kColsPerPass + c_in_pass;
+        const int n = n0 + wn * WTN + j * 32 + c;
+        const float4 lo = *reinterpret_cast<const float4 *>(area + c * kColPitch + r0);
+        const float4 hi = *reinterpret_cast<const float4 *>(area + c * kColPitch + r0 + 4);
+        if (m < g.M && n < g.N) {
+          uint16_t *p = Cz + m + (long)n * g.ldc;
+          float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+          Pack8 out;
+          if (g.accumulate) {
+            Pack8 old;
+            old.v = *reinterpret_cast<const uint4v *>(p);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] += load_c<BF16>(&old.h[e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) out.h[e] = round_c<BF16>(f[e]);
+          *reinterpret_cast<uint4v *>(p) = out.v;
+        }
+      }
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -414,6 +459,7 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
   a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
   a.rA = p.rA; a.rB = p.rB;
   a.accumulate = p.accumulate ? 1 : 0;
+  a.vec_c = reinterpret_cast<uintptr_t>(p.C) % 16 == 0 && p.M % 8 == 0 && p.ldc % 8 == 0 && p.sC % 8 == 0;
 
   auto aligned = [](const void *ptr, long ld, long s, long r) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 8 == 0 && s % 8 == 0 && r % 8 == 0;
