@@ -167,6 +167,18 @@ def _event_seconds(dev, fn, reps):
     return ms.value * 1e-3 / reps
 
 
+def _wall_seconds(dev, fn, reps):
+    """Average seconds of one blocking fn() (a call that waits for the device itself) by the host clock."""
+    for _ in range(2):
+        fn()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    dev.sync()
+    return (time.perf_counter() - t0) / reps
+
+
 def measure_pointwise(reps=20):
     """Streaming rate of the elementwise kernels: algorithmic bytes (every operand the
     operation needs read once, every result written once, a gradient read and written)
@@ -249,6 +261,30 @@ def measure_pointwise(reps=20):
                   % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
                   file=sys.stderr, flush=True)
         del m, gm, logits, table, gtable, picked, half, cases
+        # random tensors (results written once) and copies between device objects on this GPU
+        # (one read, one write; to the other storage width: converted on the way)
+        n = 64 << 20
+        other = pa.HIP16(0, storage="f16") if storage == "f32" else pa.HIP(0)
+        other_item = 2 if storage == "f32" else 4
+        src = dev.new_tensor_by_constant(S([n]), 0.5)
+        cases = [
+            ("random_uniform", lambda: dev.random_uniform(S([n]), -1.0, 1.0), n * item),
+            ("random_normal", lambda: dev.random_normal(S([n]), 0.0, 1.0), n * item),
+            ("random_bernoulli", lambda: dev.random_bernoulli(S([n]), 0.5), n * item),
+            ("copy_tensor_same_storage", lambda: dev.copy_tensor(src), 2 * n * item),
+            # to another device object: the call drains both streams itself, so the host clock times it
+            ("copy_tensor_to_" + ("f16" if storage == "f32" else "f32"), lambda: other.copy_tensor(src),
+             n * (item + other_item)),
+        ]
+        for name, fn, nbytes in cases:
+            sec = (_wall_seconds if name.startswith("copy_tensor_to") else _event_seconds)(dev, fn, reps)
+            out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
+                        "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
+            print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
+                  % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
+                  file=sys.stderr, flush=True)
+        del src, cases
+        other.close()
         dev.close()
     return out
 

@@ -59,12 +59,21 @@ template <typename T, Draw DRAW>
 __global__ __launch_bounds__(kBlock) void random_kernel(T *y, size_t n, uint64_t seed, uint64_t offset, float p0,
                                                          float p1) {
   const size_t blocks = (n + 3) / 4;
+  const bool aligned = reinterpret_cast<uintptr_t>(y) % (4 * sizeof(T)) == 0;
   for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < blocks; q += (size_t)gridDim.x * kBlock) {
     const Block b = philox4x32_10(offset + q, seed);
+    // a block's four results leave as one store (y is aligned to four elements); the last block may be short
+    struct alignas(4 * sizeof(T)) Quad {
+      T v[4];
+    } out;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const size_t i = q * 4 + e;
-      if (i < n) y[i] = from_f32<T>(draw<DRAW>(b, e, p0, p1));
+    for (int e = 0; e < 4; ++e) out.v[e] = from_f32<T>(draw<DRAW>(b, e, p0, p1));
+    if (q * 4 + 4 <= n && aligned) {
+      *reinterpret_cast<Quad *>(y + q * 4) = out;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (q * 4 + e < n) y[q * 4 + e] = out.v[e];
     }
   }
 }
