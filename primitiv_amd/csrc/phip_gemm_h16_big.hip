@@ -83,29 +83,48 @@ __device__ inline uint32_t round_c(float x) {
 // before the LDS pass, added in fp32 and rounded once.  M is a multiple of 8
 // and C is 16-byte aligned (checked by the dispatcher), so a lane's 8 rows are
 // either all inside the matrix or all outside.
-template <bool BF16>
+//
+// The area holds column c as 128 floats; row r of column c sits at position
+//   r ^ (4 * bit 6 of r) ^ (32 * bit 2 of c).
+// The first term makes the two 16-byte halves of rows 64..127 change places,
+// so that the 16 lanes of one read instruction (8 rows = 32 bytes apart) cover
+// all banks; the second moves the columns the upper half wave writes (4 further
+// on) to the other half of the banks.  Both are constants of a lane's address.
+//
+// FULL: the block lies inside the matrix, no lane is masked and the addresses
+// step by a constant; otherwise every access is checked on its own.
+template <bool BF16, bool ACC, bool FULL>
 __device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, int row0, int col0, int lane, int M,
-                                          int N, const float16v (&acc)[4][4], int accumulate) {
+                                          int N, const float16v (&acc)[4][4]) {
   const int mc = lane & 15, cq = lane >> 4;
   const int m = row0 + 8 * mc;
-  // lanes 8..15 of each group of 16 read their two 16-byte halves in the other
-  // order, which spreads a 16-lane read over all banks
-  const bool flip = (mc & 8) != 0;
+  const int flip = mc >> 3;  // rows 64..127: halves swapped
+  // write side: rows 32 i + lane % 32 of columns 32 jl + 8 (v / 4) + 4 (lane / 32) + v % 4
+  float *wbase[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    wbase[i] = area + (4 * (lane >> 5)) * 128 + ((32 * i + (lane & 31)) ^ (4 * (i >> 1)) ^ (32 * (lane >> 5)));
+  // read side: column 4 it + cq, rows 8 mc .. 8 mc + 7
+  const float *reven = area + cq * 128 + 8 * mc;               // even it
+  const float *rodd = area + cq * 128 + 8 * (mc ^ 4);          // odd it
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    uint16_t *p[16];
-    uint32_t ok = 0;
+    uint16_t *p0 = Cz + m + (long)(col0 + 64 * h + cq) * ldc;
+    uint32_t ok = 0xffffu;
+    if constexpr (!FULL) {
+      ok = 0;
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int n = col0 + 64 * h + 4 * it + cq;
-      const bool in = m < M && n < N;
-      ok |= (in ? 1u : 0u) << it;
-      p[it] = in ? Cz + m + (long)n * ldc : Cz;   // outside: read the origin, store nothing
+      for (int it = 0; it < 16; ++it)
+        ok |= (m < M && col0 + 64 * h + 4 * it + cq < N ? 1u : 0u) << it;
     }
+    auto live = [&](int it) { return FULL || ((ok >> it) & 1u); };
     uint4v old[16];
-    if (accumulate) {
+    if constexpr (ACC) {
 #pragma unroll
-      for (int it = 0; it < 16; ++it) old[it] = *reinterpret_cast<const uint4v *>(p[it]);
+      for (int it = 0; it < 16; ++it) {
+        old[it] = uint4v{0, 0, 0, 0};
+        if (live(it)) old[it] = *reinterpret_cast<const uint4v *>(p0 + (long)(4 * it) * ldc);
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -113,27 +132,28 @@ __device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, i
       for (int jl = 0; jl < 2; ++jl)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          area[(32 * jl + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4)) * 128 + 32 * i + (lane & 31)] =
-              acc[i][2 * h + jl][v];
+          wbase[i][(32 * jl + 8 * (v / 4) + (v % 4)) * 128] = acc[i][2 * h + jl][v];
+    float4 lo[16], hi[16];
 #pragma unroll
     for (int it = 0; it < 16; ++it) {
-      const float4 *src = reinterpret_cast<const float4 *>(area + (4 * it + cq) * 128 + 8 * mc);
-      const float4 first = src[flip ? 1 : 0];
-      const float4 second = src[flip ? 0 : 1];
-      const float4 lo = flip ? second : first;
-      const float4 hi = flip ? first : second;
-      float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      const float4 *src = reinterpret_cast<const float4 *>(((it & 1) ? rodd : reven) + 4 * it * 128);
+      lo[it] = src[flip];
+      hi[it] = src[flip ^ 1];
+    }
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      float f[8] = {lo[it].x, lo[it].y, lo[it].z, lo[it].w, hi[it].x, hi[it].y, hi[it].z, hi[it].w};
       uint4v out;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float x0 = f[2 * e], x1 = f[2 * e + 1];
-        if (accumulate) {
+        if constexpr (ACC) {
           x0 += widen<BF16>(old[it][e] & 0xffffu);
           x1 += widen<BF16>(old[it][e] >> 16);
         }
         out[e] = round_c<BF16>(x0) | (round_c<BF16>(x1) << 16);
       }
-      if ((ok >> it) & 1u) *reinterpret_cast<uint4v *>(p[it]) = out;
+      if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(4 * it) * ldc) = out;
     }
   }
 }
@@ -378,8 +398,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_h16_lds_kernel(const BigArgs
   __syncthreads();
 
   uint16_t *Cz = g.C + (long)z * g.sC;
-  emit_block_via_lds<BF16>(reinterpret_cast<float *>(lds2 + wave * kRegionBytes), Cz, g.ldc, m0 + wm * 128,
-                           n0 + wn * 128, lane, g.M, g.N, acc, g.accumulate);
+  float *area = reinterpret_cast<float *>(lds2 + wave * kRegionBytes);
+  const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
+  const bool full = row0 + 128 <= g.M && col0 + 128 <= g.N;  // the same for every lane of the wavefront
+  if (g.accumulate) {
+    if (full) emit_block_via_lds<BF16, true, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+    else emit_block_via_lds<BF16, true, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+  } else {
+    if (full) emit_block_via_lds<BF16, false, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+    else emit_block_via_lds<BF16, false, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+  }
 }
 
 template <bool BF16>
