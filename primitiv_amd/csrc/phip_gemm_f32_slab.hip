@@ -261,7 +261,7 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   const long total_ktiles = (long)ktiles_per_r * p.rbatch;
   const long tiles = (long)((p.M + TBM - 1) / TBM) * p.batch;
   const int cus = ctx->prop.multiProcessorCount;
-  if (a_bytes * p.rbatch * p.batch < (8L << 20) || total_ktiles > 0x7fffffffL || tiles > 0x3fffffffL) return PHIP_OK;
+  if (a_bytes * p.rbatch * p.batch < kStreamedOperandBytes || total_ktiles > 0x7fffffffL || tiles > 0x3fffffffL) return PHIP_OK;
   // two workgroups fit a compute unit: fill those places at most once (a workgroup that has to wait for
   // a place doubles the launch's duration), at least eight stages each
   long splits = 2L * cus / tiles;

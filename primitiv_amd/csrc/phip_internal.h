@@ -126,6 +126,13 @@ int gemm_f32_direct(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_slab(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_rankk(phip_ctx *ctx, const Gemm &g, bool *handled);
+// Two independent accumulating products (outputs do not overlap) in one launch,
+// for problems so small that a launch is mostly its fixed latency.  Sets
+// *handled when it launched both; otherwise nothing has been done.
+int gemm_f32_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *handled);
+// An operand of at least this many bytes, read once against few output columns,
+// is worth the streaming kernel (gemm_f32_slab).
+constexpr long kStreamedOperandBytes = 8L << 20;
 int gemm_h16(phip_ctx *ctx, const Gemm &g, Elem elem);
 int gemm_h16_big(phip_ctx *ctx, const Gemm &g, Elem elem, bool *handled);
 

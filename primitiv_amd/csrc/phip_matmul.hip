@@ -85,8 +85,6 @@ static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, con
     p.K = (int)(dk * bb);  // contraction over (column, sample)
     p.batch = 1;
   }
-  rc = gemm_dispatch(ctx, p, elem);
-  if (rc != PHIP_OK) return rc;
 
   // gb[dj x dk] += a^T . gy : A = a^T with element (m, k) at k + m*di, B = gy
   // with element (k, n) at k + n*di (both k-contiguous).
@@ -114,6 +112,19 @@ static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, con
     q.N = (int)(dk * bb);
     q.batch = 1;
   }
+
+  // Small products whose outputs do not overlap share one launch.
+  if (elem == Elem::F32) {
+    const char *ga0 = static_cast<const char *>(ga), *gb0 = static_cast<const char *>(gb);
+    const size_t ga_bytes = sizeof(float) * (size_t)di * dj * ba, gb_bytes = sizeof(float) * (size_t)dj * dk * bb;
+    if (ga0 + ga_bytes <= gb0 || gb0 + gb_bytes <= ga0) {
+      bool handled = false;
+      rc = gemm_f32_pair(ctx, p, q, &handled);
+      if (rc != PHIP_OK || handled) return rc;
+    }
+  }
+  rc = gemm_dispatch(ctx, p, elem);
+  if (rc != PHIP_OK) return rc;
   return gemm_dispatch(ctx, q, elem);
 }
 

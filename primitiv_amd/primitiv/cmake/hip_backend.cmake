@@ -40,6 +40,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_slab.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_rankk.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_pair.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16_big.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_matmul.hip

@@ -250,6 +250,56 @@ def test_streamed_operand_f32(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(y2, ry) <= F32_TOL
 
 
+# both gradient products of a small matmul leave in one launch when their outputs do not
+# overlap: the dense layer, the recurrent gate (a rank-K update by staged 64 x 64 tiles
+# beside a long-K product split between workgroups), ragged edges, a contraction over
+# the minibatch, per-sample products
+PAIRED_F32 = [  # di, dj, dk, ba, bb
+    (256, 784, 1, 1, 128),
+    (2048, 512, 1, 1, 64),
+    (2052, 516, 1, 1, 60),
+    (512, 96, 260, 1, 1),
+    (64, 64, 8, 9, 1),
+    (132, 260, 24, 6, 6),
+    (1024, 1024, 1, 1, 8),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", PAIRED_F32)
+def test_paired_gradient_products_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di * 3 + dj + dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    _, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(ga, rga) <= F32_TOL
+    assert norm_rel_err(gb, rgb) <= F32_TOL
+
+
+def test_gradients_into_one_buffer(dev):
+    # ga and gb may be the same memory (the gradient of x.x for a square x): the two
+    # products must then add one after the other, not race
+    from primitiv_amd import _lib
+    n = 96
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(n * n).astype(np.float32)
+    b = rng.standard_normal(n * n).astype(np.float32)
+    gy = rng.standard_normal(n * n).astype(np.float32)
+    g0 = rng.standard_normal(n * n).astype(np.float32)
+    sh = pa.Shape([n, n])
+    ta, tb, tgy, tg = (dev.new_tensor_by_vector(sh, v) for v in (a, b, gy, g0))
+    rc = _lib.lib().phip_matmul_bw_f32(dev.ctx(), ta.handle(), tb.handle(), tgy.handle(), tg.handle(), tg.handle(),
+                                       n, n, n, 1, 1)
+    assert rc == 0
+    zero = np.zeros(n * n, np.float32)
+    rga, rgb = oracle.matmul_bw(a, b, gy, g0, zero, n, n, n, 1, 1, 4)
+    assert norm_rel_err(tg.to_vector(), rga + rgb) <= F32_TOL
+
+
 # an overwriting product with few output tiles and a long K is cut between workgroups
 # that meet through partial tiles, summed in a fixed order by whichever finishes last:
 # right, and the same bits on every run
