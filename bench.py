@@ -289,6 +289,54 @@ def measure_pointwise(reps=20):
     return out
 
 
+def measure_conv(reps=10):
+    """conv2d (2 * outputs * taps flops forward, twice that backward, against the MFMA peak of the
+    storage type) and max_pool2d (x read, y written; backward: x, y, gy read, gx read and written,
+    against the HBM peak) on image-model layer shapes."""
+    S = pa.Shape
+    out = []
+    layers = [  # name, x dims, w dims, minibatch, (pad0, pad1, str0, str1, dil0, dil1)
+        ("vgg16_conv1_2", [224, 224, 64], [3, 3, 64, 64], 8, (1, 1, 1, 1, 1, 1)),
+        ("vgg16_conv4_2", [28, 28, 512], [3, 3, 512, 512], 32, (1, 1, 1, 1, 1, 1)),
+        ("pointwise_1x1", [56, 56, 256], [1, 1, 256, 64], 32, (0, 0, 1, 1, 1, 1)),
+        ("mnist_conv1", [28, 28, 1], [5, 5, 1, 8], 200, (2, 2, 1, 1, 1, 1)),
+    ]
+    for storage, item in (("f32", 4), ("f16", 2)):
+        dev = pa.HIP(0, rng_seed=1) if storage == "f32" else pa.HIP16(0, rng_seed=1, storage=storage)
+        for name, xd, wd, bs, a in layers:
+            x = dev.random_normal(S(xd, bs), 0.0, 1.0)
+            w = dev.random_normal(S(wd), 0.0, 0.05)
+            y = dev.conv2d_fw(x, w, *a)
+            gx = dev.new_tensor_by_constant(x.shape(), 0.0)
+            gw = dev.new_tensor_by_constant(w.shape(), 0.0)
+            flops = 2.0 * y.shape().size() * wd[0] * wd[1] * wd[2]
+            for tag, fn, work in (("fw", lambda: dev.conv2d_fw(x, w, *a), flops),
+                                  ("bw", lambda: dev.conv2d_bw(x, w, y, y, *a, gx, gw), 2 * flops)):
+                sec = _event_seconds(dev, fn, reps)
+                out.append({"kernel": "conv2d_%s_%s" % (tag, name), "dtype": storage, "flops": work, "us": sec * 1e6,
+                            "tflops": work / sec / 1e12, "frac_mfma_peak": work / sec / 1e12 / PEAK_TFLOPS[storage]})
+                print("# %-28s %s  %9.1f us  %7.1f TFLOP/s (%.1f%% of MFMA peak)"
+                      % (out[-1]["kernel"], storage, sec * 1e6, out[-1]["tflops"], 100 * out[-1]["frac_mfma_peak"]),
+                      file=sys.stderr, flush=True)
+            del x, w, y, gx, gw
+        x = dev.random_normal(S([224, 224, 64], 8), 0.0, 1.0)
+        a = (2, 2, 0, 0, 2, 2)
+        y = dev.max_pool2d_fw(x, *a)
+        gx = dev.new_tensor_by_constant(x.shape(), 0.0)
+        nx, ny = x.shape().size() * item, y.shape().size() * item
+        for tag, fn, nbytes in (("fw", lambda: dev.max_pool2d_fw(x, *a), nx + ny),
+                                ("bw", lambda: dev.max_pool2d_bw(x, y, y, *a, gx), 3 * nx + 2 * ny)):
+            sec = _event_seconds(dev, fn, reps)
+            out.append({"kernel": "max_pool2d_%s_2x2" % tag, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
+                        "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
+            print("# %-28s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
+                  % (out[-1]["kernel"], storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
+                  file=sys.stderr, flush=True)
+        del x, y, gx
+        dev.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,6 +349,8 @@ def main():
                          "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--pointwise", action="store_true",
                     help="measure the elementwise kernels' streaming rates instead of the matmul workloads")
+    ap.add_argument("--conv", action="store_true",
+                    help="measure conv2d and max_pool2d on image-model layer shapes instead of the matmul workloads")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path "
@@ -308,6 +358,11 @@ def main():
     if args.pointwise:
         print(json.dumps({"metric": "elementwise kernels, algorithmic GB/s", "unit": "GB/s", "n_gpus": 1,
                           "peak": PEAK_HBM_GBS, "data": "synthetic", "kernels": measure_pointwise()}))
+        return
+
+    if args.conv:
+        print(json.dumps({"metric": "conv2d TFLOP/s, max_pool2d algorithmic GB/s", "n_gpus": 1,
+                          "data": "synthetic", "kernels": measure_conv()}))
         return
 
     if args.traffic_calibration:

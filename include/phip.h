@@ -493,6 +493,60 @@ int phip_random_log_normal_f16(phip_ctx *ctx, uint64_t seed, uint64_t offset, fl
 int phip_random_log_normal_bf16(phip_ctx *ctx, uint64_t seed, uint64_t offset, float mean, float sd,
                                void *y, size_t n);
 
+/* ---- convolution and pooling -----------------------------------------------
+ * conv2d: x is x0 x x1 x c per sample (first dimension contiguous), w is
+ * w0 x w1 x c x oc, y is y0 x y1 x oc with y0 = (x0 + 2 pad0 - ((w0-1) dil0 + 1))
+ * / str0 + 1 and y1 likewise (primitiv/core/shape_ops.cc:162-187); bx and bw
+ * are the minibatch sizes of x and w (equal, or 1 = shared by all samples).
+ * A true convolution: the tap at window offset (i, j) meets kernel element
+ * (w0-1-i, w1-1-j).  Forward overwrites y; backward adds to gx (shape of x) and
+ * gw (shape of w), a shared operand's gradient collecting every sample.
+ * Scratch comes from the context's pool.
+ * Reference: conv2d_fw_impl / conv2d_bw_impl (primitiv/devices/naive/ops/
+ * conv2d.cc:9-151 for the arithmetic, primitiv/devices/cuda/ops/conv2d.cu:11-198
+ * for the device interface). */
+int phip_conv2d_fw_f32(phip_ctx *ctx, const float *x, const float *w, float *y, uint32_t x0, uint32_t x1,
+    uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw, uint32_t pad0, uint32_t pad1,
+    uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+int phip_conv2d_bw_f32(phip_ctx *ctx, const float *x, const float *w, const float *gy, float *gx, float *gw,
+    uint32_t x0, uint32_t x1, uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw,
+    uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+int phip_conv2d_fw_f16(phip_ctx *ctx, const void *x, const void *w, void *y, uint32_t x0, uint32_t x1,
+    uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw, uint32_t pad0, uint32_t pad1,
+    uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+int phip_conv2d_bw_f16(phip_ctx *ctx, const void *x, const void *w, const void *gy, void *gx, void *gw,
+    uint32_t x0, uint32_t x1, uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw,
+    uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+int phip_conv2d_fw_bf16(phip_ctx *ctx, const void *x, const void *w, void *y, uint32_t x0, uint32_t x1,
+    uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw, uint32_t pad0, uint32_t pad1,
+    uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+int phip_conv2d_bw_bf16(phip_ctx *ctx, const void *x, const void *w, const void *gy, void *gx, void *gw,
+    uint32_t x0, uint32_t x1, uint32_t c, uint32_t w0, uint32_t w1, uint32_t oc, uint32_t bx, uint32_t bw,
+    uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1, uint32_t dil0, uint32_t dil1);
+
+/* max_pool2d over `repeat` planes of x0 x x1 (channels times minibatch): y is
+ * y0 x y1 per plane with y0 = (x0 + 2 pad0 - win0) / str0 + 1 and y1 likewise
+ * (shape_ops.cc:189-213); padding never wins.  Backward adds gy to the FIRST
+ * element of each window (second window axis outer, first inner) that equals
+ * y; the same bits on every run.
+ * Reference: max_pool2d_fw_impl / max_pool2d_bw_impl (primitiv/devices/naive/ops/
+ * max_pool2d.cc:9-113, primitiv/devices/cuda/ops/max_pool2d.cu:11-117). */
+int phip_max_pool2d_fw_f32(phip_ctx *ctx, const float *x, float *y, uint32_t x0, uint32_t x1, uint32_t repeat,
+    uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1);
+int phip_max_pool2d_bw_f32(phip_ctx *ctx, const float *x, const float *y, const float *gy, float *gx,
+    uint32_t x0, uint32_t x1, uint32_t repeat, uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1,
+    uint32_t str0, uint32_t str1);
+int phip_max_pool2d_fw_f16(phip_ctx *ctx, const void *x, void *y, uint32_t x0, uint32_t x1, uint32_t repeat,
+    uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1);
+int phip_max_pool2d_bw_f16(phip_ctx *ctx, const void *x, const void *y, const void *gy, void *gx, uint32_t x0,
+    uint32_t x1, uint32_t repeat, uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1, uint32_t str0,
+    uint32_t str1);
+int phip_max_pool2d_fw_bf16(phip_ctx *ctx, const void *x, void *y, uint32_t x0, uint32_t x1, uint32_t repeat,
+    uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1, uint32_t str0, uint32_t str1);
+int phip_max_pool2d_bw_bf16(phip_ctx *ctx, const void *x, const void *y, const void *gy, void *gx, uint32_t x0,
+    uint32_t x1, uint32_t repeat, uint32_t win0, uint32_t win1, uint32_t pad0, uint32_t pad1, uint32_t str0,
+    uint32_t str1);
+
 /* ---- timing ---------------------------------------------------------------
  * No counterpart in the reference (it has no profiling facility); events are
  * recorded on the context's stream so they bracket exactly the kernels the

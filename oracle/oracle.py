@@ -25,6 +25,7 @@ __all__ = [
     "transpose_bw", "permute_dims_fw", "permute_dims_bw", "flip_fw", "flip_bw", "reduce_fw",
     "extremum_bw", "arg_extremum", "broadcast_fw",
     "RANDOM_KINDS", "philox4x32_10", "random",
+    "shape_conv2d", "shape_pool2d", "conv2d_fw", "conv2d_bw", "max_pool2d_fw", "max_pool2d_bw",
 ]
 
 _F = ctypes.POINTER(ctypes.c_float)
@@ -107,6 +108,18 @@ def lib():
         l.ref_philox4x32_10.argtypes = [_D, _D, _D]
         l.ref_philox4x32_10.restype = None
         l.ref_random.argtypes = [_I, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float, _F, _Z]
+        l.ref_shape_conv2d.argtypes = [_U] * 15 + [_D, _D]
+        l.ref_shape_conv2d.restype = ctypes.c_int
+        l.ref_shape_pool2d.argtypes = [_U] * 8 + [_D]
+        l.ref_shape_pool2d.restype = ctypes.c_int
+        l.ref_conv2d_fw.argtypes = [_F, _F, _F] + [_U] * 14
+        l.ref_conv2d_fw.restype = None
+        l.ref_conv2d_bw.argtypes = [_F, _F, _F, _F, _F] + [_U] * 14
+        l.ref_conv2d_bw.restype = None
+        l.ref_max_pool2d_fw.argtypes = [_F, _F] + [_U] * 9
+        l.ref_max_pool2d_fw.restype = None
+        l.ref_max_pool2d_bw.argtypes = [_F, _F, _F, _F] + [_U] * 9
+        l.ref_max_pool2d_bw.restype = None
         _lib = l
     return _lib
 
@@ -512,3 +525,70 @@ def random(kind, seed, offset, p0, p1, n):
     y = np.empty(n, dtype=np.float32)
     _ok(lib().ref_random(RANDOM_KINDS.index(kind), seed, offset, p0, p1, _p(y), n), kind)
     return y
+
+
+# ---- convolution and pooling (ref_conv_pool.c) ---------------------------------
+def _pad(dims, n):
+    dims = [int(d) for d in dims]
+    return dims + [1] * (n - len(dims))
+
+
+def shape_conv2d(x_dims, bx, w_dims, bw, pad0, pad1, str0, str1, dil0, dil1):
+    """(dims, batch) of conv2d's result; ValueError for arguments the reference rejects
+    (shape_ops.cc:162-187)."""
+    if len(x_dims) > 3 or len(w_dims) > 4:
+        raise ValueError("Invalid arguments to calculate a convolution")
+    x, w = _pad(x_dims, 3), _pad(w_dims, 4)
+    dims, batch = (_U * 3)(), (_U * 1)()
+    if lib().ref_shape_conv2d(x[0], x[1], x[2], bx, w[0], w[1], w[2], w[3], bw, pad0, pad1, str0, str1, dil0, dil1,
+                              dims, batch):
+        raise ValueError("Invalid arguments to calculate a convolution")
+    return list(dims), int(batch[0])
+
+
+def shape_pool2d(x_dims, win0, win1, pad0, pad1, str0, str1):
+    """dims of max_pool2d's result (the minibatch is x's); ValueError as shape_ops.cc:189-213."""
+    if len(x_dims) > 3:
+        raise ValueError("Invalid arguments to calculate a pooling")
+    x = _pad(x_dims, 3)
+    dims = (_U * 2)()
+    if lib().ref_shape_pool2d(x[0], x[1], win0, win1, pad0, pad1, str0, str1, dims):
+        raise ValueError("Invalid arguments to calculate a pooling")
+    return [int(dims[0]), int(dims[1]), x[2]]
+
+
+def conv2d_fw(x, w, x_dims, bx, w_dims, bw, pad0, pad1, str0, str1, dil0, dil1):
+    x, w = _f32(x), _f32(w)
+    xd, wd = _pad(x_dims, 3), _pad(w_dims, 4)
+    yd, bs = shape_conv2d(x_dims, bx, w_dims, bw, pad0, pad1, str0, str1, dil0, dil1)
+    y = np.empty(int(np.prod(yd)) * bs, dtype=np.float32)
+    lib().ref_conv2d_fw(_p(x), _p(w), _p(y), xd[0], xd[1], xd[2], wd[0], wd[1], wd[3], bx, bw, pad0, pad1, str0, str1,
+                        dil0, dil1)
+    return y
+
+
+def conv2d_bw(x, w, gy, gx, gw, x_dims, bx, w_dims, bw, pad0, pad1, str0, str1, dil0, dil1):
+    """(gx, gw) after the gradients have been added to copies of the given ones."""
+    x, w, gy = _f32(x), _f32(w), _f32(gy)
+    gx, gw = _f32(gx).copy(), _f32(gw).copy()
+    xd, wd = _pad(x_dims, 3), _pad(w_dims, 4)
+    lib().ref_conv2d_bw(_p(x), _p(w), _p(gy), _p(gx), _p(gw), xd[0], xd[1], xd[2], wd[0], wd[1], wd[3], bx, bw, pad0,
+                        pad1, str0, str1, dil0, dil1)
+    return gx, gw
+
+
+def max_pool2d_fw(x, x_dims, bs, win0, win1, pad0, pad1, str0, str1):
+    x = _f32(x)
+    xd = _pad(x_dims, 3)
+    yd = shape_pool2d(x_dims, win0, win1, pad0, pad1, str0, str1)
+    y = np.empty(yd[0] * yd[1] * xd[2] * bs, dtype=np.float32)
+    lib().ref_max_pool2d_fw(_p(x), _p(y), xd[0], xd[1], xd[2] * bs, win0, win1, pad0, pad1, str0, str1)
+    return y
+
+
+def max_pool2d_bw(x, y, gy, gx, x_dims, bs, win0, win1, pad0, pad1, str0, str1):
+    x, y, gy = _f32(x), _f32(y), _f32(gy)
+    gx = _f32(gx).copy()
+    xd = _pad(x_dims, 3)
+    lib().ref_max_pool2d_bw(_p(x), _p(y), _p(gy), _p(gx), xd[0], xd[1], xd[2] * bs, win0, win1, pad0, pad1, str0, str1)
+    return gx

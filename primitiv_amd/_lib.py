@@ -182,6 +182,18 @@ SIGNATURES = {
     "phip_matmul_bw_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_bw_f16": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_bw_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_conv2d_fw_f32": [_vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_conv2d_bw_f32": [_vp, _vp, _vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_max_pool2d_fw_f32": [_vp, _vp, _vp] + [_u32] * 9,
+    "phip_max_pool2d_bw_f32": [_vp, _vp, _vp, _vp, _vp] + [_u32] * 9,
+    "phip_conv2d_fw_f16": [_vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_conv2d_bw_f16": [_vp, _vp, _vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_max_pool2d_fw_f16": [_vp, _vp, _vp] + [_u32] * 9,
+    "phip_max_pool2d_bw_f16": [_vp, _vp, _vp, _vp, _vp] + [_u32] * 9,
+    "phip_conv2d_fw_bf16": [_vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_conv2d_bw_bf16": [_vp, _vp, _vp, _vp, _vp, _vp] + [_u32] * 14,
+    "phip_max_pool2d_fw_bf16": [_vp, _vp, _vp] + [_u32] * 9,
+    "phip_max_pool2d_bw_bf16": [_vp, _vp, _vp, _vp, _vp] + [_u32] * 9,
     "phip_event_create": [_vp, _pp],
     "phip_event_destroy": [_vp],
     "phip_event_record": [_vp, _vp],

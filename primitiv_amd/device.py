@@ -123,6 +123,28 @@ class shape_ops:
         return Shape([l[0], r[1]], max(l.batch(), r.batch()))
 
     @staticmethod
+    def conv2d(x, w, padding0, padding1, stride0, stride1, dilation0, dilation1):
+        # shape_ops.cc:162-187
+        x0, x1 = x[0] + 2 * padding0, x[1] + 2 * padding1
+        w0, w1 = (w[0] - 1) * dilation0 + 1, (w[1] - 1) * dilation1 + 1
+        if (x.depth() > 3 or w.depth() > 4 or x0 < w0 or x1 < w1 or x[2] != w[2]
+                or not x.has_compatible_batch(w) or stride0 == 0 or stride1 == 0
+                or dilation0 == 0 or dilation1 == 0):
+            raise Error("Invalid arguments to calculate a convolution: %s, %s, %d, %d, %d, %d, %d, %d"
+                        % (x.to_string(), w.to_string(), padding0, padding1, stride0, stride1, dilation0, dilation1))
+        return Shape([(x0 - w0) // stride0 + 1, (x1 - w1) // stride1 + 1, w[3]], max(x.batch(), w.batch()))
+
+    @staticmethod
+    def pool2d(x, window0, window1, padding0, padding1, stride0, stride1):
+        # shape_ops.cc:189-213
+        x0, x1 = x[0] + 2 * padding0, x[1] + 2 * padding1
+        if (x.depth() > 3 or x0 < window0 or x1 < window1 or window0 == 0 or window1 == 0
+                or stride0 == 0 or stride1 == 0):
+            raise Error("Invalid arguments to calculate a pooling: %s, %d, %d, %d, %d, %d, %d"
+                        % (x.to_string(), window0, window1, padding0, padding1, stride0, stride1))
+        return Shape([(x0 - window0) // stride0 + 1, (x1 - window1) // stride1 + 1, x[2]], x.batch())
+
+    @staticmethod
     def batch_sum(x):
         return x.resize_batch(1)
 
@@ -500,6 +522,59 @@ class HIP:
         pga, pgb = ga.mutable_handle(), gb.mutable_handle()
         _lib.call("phip_matmul_bw_" + self._SUFFIX, self._ctx, a.handle(), b.handle(),
                   gy.handle(), pga, pgb, sa[0], sa[1], sb[1], sa.batch(), sb.batch())
+
+    # -- convolution and pooling -------------------------------------------
+    def conv2d_fw(self, x, w, padding0, padding1, stride0, stride1, dilation0, dilation1):
+        # device.cc:420-433
+        self._check_device(x)
+        self._check_device(w)
+        args = (padding0, padding1, stride0, stride1, dilation0, dilation1)
+        y = self.new_raw_tensor(shape_ops.conv2d(x.shape(), w.shape(), *args))
+        sx, sw = x.shape(), w.shape()
+        _lib.call("phip_conv2d_fw_" + self._SUFFIX, self._ctx, x.handle(), w.handle(), y.mutable_handle(),
+                  sx[0], sx[1], sx[2], sw[0], sw[1], sw[3], sx.batch(), sw.batch(), *args)
+        return y
+
+    def conv2d_bw(self, x, w, y, gy, padding0, padding1, stride0, stride1, dilation0, dilation1, gx, gw):
+        # device.cc:455-491
+        for t in (x, w, y, gy, gx, gw):
+            self._check_device(t)
+        args = (padding0, padding1, stride0, stride1, dilation0, dilation1)
+        if (x.shape() != gx.shape() or w.shape() != gw.shape() or y.shape() != gy.shape()
+                or y.shape() != shape_ops.conv2d(x.shape(), w.shape(), *args)):
+            raise Error("Shape mismatched at conv2d_bw. x.shape: %s, w.shape: %s, y.shape: %s, gy.shape: %s, "
+                        "gx.shape: %s, gw.shape: %s, padding0: %d, padding1: %d, stride0: %d, stride1: %d, "
+                        "dilation0: %d, dilation1: %d"
+                        % (tuple(t.shape().to_string() for t in (x, w, y, gy, gx, gw)) + args))
+        sx, sw = x.shape(), w.shape()
+        pgx, pgw = gx.mutable_handle(), gw.mutable_handle()
+        _lib.call("phip_conv2d_bw_" + self._SUFFIX, self._ctx, x.handle(), w.handle(), gy.handle(), pgx, pgw,
+                  sx[0], sx[1], sx[2], sw[0], sw[1], sw[3], sx.batch(), sw.batch(), *args)
+
+    def max_pool2d_fw(self, x, window0, window1, padding0, padding1, stride0, stride1):
+        # device.cc:435-446
+        self._check_device(x)
+        args = (window0, window1, padding0, padding1, stride0, stride1)
+        y = self.new_raw_tensor(shape_ops.pool2d(x.shape(), *args))
+        sx = x.shape()
+        _lib.call("phip_max_pool2d_fw_" + self._SUFFIX, self._ctx, x.handle(), y.mutable_handle(), sx[0], sx[1],
+                  sx.size() // (sx[0] * sx[1]), *args)
+        return y
+
+    def max_pool2d_bw(self, x, y, gy, window0, window1, padding0, padding1, stride0, stride1, gx):
+        # device.cc:493-522
+        for t in (x, y, gy, gx):
+            self._check_device(t)
+        args = (window0, window1, padding0, padding1, stride0, stride1)
+        if (x.shape() != gx.shape() or y.shape() != gy.shape()
+                or y.shape() != shape_ops.pool2d(x.shape(), *args)):
+            raise Error("Shape mismatched at max_pool2d_bw. x.shape: %s, y.shape: %s, gy.shape: %s, gx.shape: %s, "
+                        "window0: %d, window1: %d, padding0: %d, padding1: %d, stride0: %d, stride1: %d"
+                        % (tuple(t.shape().to_string() for t in (x, y, gy, gx)) + args))
+        sx = x.shape()
+        pgx = gx.mutable_handle()
+        _lib.call("phip_max_pool2d_bw_" + self._SUFFIX, self._ctx, x.handle(), y.handle(), gy.handle(), pgx, sx[0],
+                  sx[1], sx.size() // (sx[0] * sx[1]), *args)
 
     def inplace_add(self, x, y):
         # device.cc:692-703

@@ -245,11 +245,6 @@ HIP16::HIP16(std::uint32_t device_id, std::uint32_t rng_seed)
 HIP16::HIP16(std::uint32_t device_id)
 : HIP(device_id, std::random_device()(), Storage::F16) {}
 
-void HIP::unsupported(const char *op) {
-  PRIMITIV_THROW_NOT_IMPLEMENTED_WITH_MESSAGE(
-      "devices::HIP implements the matmul path only; `" << op << "` is not available.");
-}
-
 void HIP::dump_description() const {
   char buf[2048];
   PHIP_CALL(::phip_describe(ctx_, buf, sizeof(buf)));
@@ -763,6 +758,87 @@ PHIP_DEF_AB(pow, PHIP_POW)
 #undef PHIP_DEF_CONST
 #undef PHIP_DEF_SCALAR
 #undef PHIP_DEF_AB
+
+// ---- convolution and pooling --------------------------------------------------
+
+void HIP::conv2d_fw_impl(
+    const Tensor &x, const Tensor &w, std::uint32_t padding0, std::uint32_t padding1, std::uint32_t stride0,
+    std::uint32_t stride1, std::uint32_t dilation0, std::uint32_t dilation1, Tensor &y) {
+  const Shape &sx = x.shape();
+  const Shape &sw = w.shape();
+  void *py = get_mutable_handle(y);
+  const void *px = get_handle(x), *pw = get_handle(w);
+#define PHIP_CONV_FW(SUF, CPTR, PTR)                                                                        \
+  PHIP_CALL(::phip_conv2d_fw_##SUF(ctx_, static_cast<CPTR>(px), static_cast<CPTR>(pw), static_cast<PTR>(py), \
+                                   sx[0], sx[1], sx[2], sw[0], sw[1], sw[3], sx.batch(), sw.batch(),         \
+                                   padding0, padding1, stride0, stride1, dilation0, dilation1))
+  switch (storage_) {
+    case Storage::F32: PHIP_CONV_FW(f32, const float *, float *); break;
+    case Storage::F16: PHIP_CONV_FW(f16, const void *, void *); break;
+    default: PHIP_CONV_FW(bf16, const void *, void *); break;
+  }
+#undef PHIP_CONV_FW
+}
+
+void HIP::conv2d_bw_impl(
+    const Tensor &x, const Tensor &w, const Tensor &, const Tensor &gy, std::uint32_t padding0,
+    std::uint32_t padding1, std::uint32_t stride0, std::uint32_t stride1, std::uint32_t dilation0,
+    std::uint32_t dilation1, Tensor &gx, Tensor &gw) {
+  const Shape &sx = x.shape();
+  const Shape &sw = w.shape();
+  // writable pointers first: taking them may clone a shared block
+  void *pgx = get_mutable_handle(gx);
+  void *pgw = get_mutable_handle(gw);
+  const void *px = get_handle(x), *pw = get_handle(w), *pgy = get_handle(gy);
+#define PHIP_CONV_BW(SUF, CPTR, PTR)                                                                          \
+  PHIP_CALL(::phip_conv2d_bw_##SUF(ctx_, static_cast<CPTR>(px), static_cast<CPTR>(pw), static_cast<CPTR>(pgy), \
+                                   static_cast<PTR>(pgx), static_cast<PTR>(pgw), sx[0], sx[1], sx[2], sw[0],   \
+                                   sw[1], sw[3], sx.batch(), sw.batch(), padding0, padding1, stride0, stride1, \
+                                   dilation0, dilation1))
+  switch (storage_) {
+    case Storage::F32: PHIP_CONV_BW(f32, const float *, float *); break;
+    case Storage::F16: PHIP_CONV_BW(f16, const void *, void *); break;
+    default: PHIP_CONV_BW(bf16, const void *, void *); break;
+  }
+#undef PHIP_CONV_BW
+}
+
+void HIP::max_pool2d_fw_impl(
+    const Tensor &x, std::uint32_t window0, std::uint32_t window1, std::uint32_t padding0, std::uint32_t padding1,
+    std::uint32_t stride0, std::uint32_t stride1, Tensor &y) {
+  const Shape &sx = x.shape();
+  const std::uint32_t repeat = sx.size() / (sx[0] * sx[1]);  // channels and samples alike
+  void *py = get_mutable_handle(y);
+  const void *px = get_handle(x);
+#define PHIP_POOL_FW(SUF, CPTR, PTR)                                                                       \
+  PHIP_CALL(::phip_max_pool2d_fw_##SUF(ctx_, static_cast<CPTR>(px), static_cast<PTR>(py), sx[0], sx[1], repeat, \
+                                       window0, window1, padding0, padding1, stride0, stride1))
+  switch (storage_) {
+    case Storage::F32: PHIP_POOL_FW(f32, const float *, float *); break;
+    case Storage::F16: PHIP_POOL_FW(f16, const void *, void *); break;
+    default: PHIP_POOL_FW(bf16, const void *, void *); break;
+  }
+#undef PHIP_POOL_FW
+}
+
+void HIP::max_pool2d_bw_impl(
+    const Tensor &x, const Tensor &y, const Tensor &gy, std::uint32_t window0, std::uint32_t window1,
+    std::uint32_t padding0, std::uint32_t padding1, std::uint32_t stride0, std::uint32_t stride1, Tensor &gx) {
+  const Shape &sx = x.shape();
+  const std::uint32_t repeat = sx.size() / (sx[0] * sx[1]);
+  void *pgx = get_mutable_handle(gx);
+  const void *px = get_handle(x), *py = get_handle(y), *pgy = get_handle(gy);
+#define PHIP_POOL_BW(SUF, CPTR, PTR)                                                                         \
+  PHIP_CALL(::phip_max_pool2d_bw_##SUF(ctx_, static_cast<CPTR>(px), static_cast<CPTR>(py), static_cast<CPTR>(pgy), \
+                                       static_cast<PTR>(pgx), sx[0], sx[1], repeat, window0, window1, padding0, \
+                                       padding1, stride0, stride1))
+  switch (storage_) {
+    case Storage::F32: PHIP_POOL_BW(f32, const float *, float *); break;
+    case Storage::F16: PHIP_POOL_BW(f16, const void *, void *); break;
+    default: PHIP_POOL_BW(bf16, const void *, void *); break;
+  }
+#undef PHIP_POOL_BW
+}
 
 }  // namespace devices
 }  // namespace primitiv

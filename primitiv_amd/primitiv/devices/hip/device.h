@@ -143,22 +143,20 @@ private:
 #undef PHIP_DECL_SCALAR
 #undef PHIP_DECL_AB
 
-  // ---- not implemented in this backend -------------------------------------
-  [[noreturn]] static void unsupported(const char *op);
-
-
-
-  void conv2d_fw_impl(const Tensor &, const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t,
-                      std::uint32_t, std::uint32_t, std::uint32_t, Tensor &) override { unsupported("conv2d_fw"); }
-  void conv2d_bw_impl(const Tensor &, const Tensor &, const Tensor &, const Tensor &, std::uint32_t,
-                      std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
-                      Tensor &, Tensor &) override { unsupported("conv2d_bw"); }
-  void max_pool2d_fw_impl(const Tensor &, std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
-                          std::uint32_t, std::uint32_t, Tensor &) override { unsupported("max_pool2d_fw"); }
-  void max_pool2d_bw_impl(const Tensor &, const Tensor &, const Tensor &, std::uint32_t, std::uint32_t,
-                          std::uint32_t, std::uint32_t, std::uint32_t, std::uint32_t,
-                          Tensor &) override { unsupported("max_pool2d_bw"); }
-
+  // ---- convolution and pooling ----------------------------------------------
+  void conv2d_fw_impl(const Tensor &x, const Tensor &w, std::uint32_t padding0, std::uint32_t padding1,
+                      std::uint32_t stride0, std::uint32_t stride1, std::uint32_t dilation0,
+                      std::uint32_t dilation1, Tensor &y) override;
+  void conv2d_bw_impl(const Tensor &x, const Tensor &w, const Tensor &y, const Tensor &gy,
+                      std::uint32_t padding0, std::uint32_t padding1, std::uint32_t stride0,
+                      std::uint32_t stride1, std::uint32_t dilation0, std::uint32_t dilation1,
+                      Tensor &gx, Tensor &gw) override;
+  void max_pool2d_fw_impl(const Tensor &x, std::uint32_t window0, std::uint32_t window1, std::uint32_t padding0,
+                          std::uint32_t padding1, std::uint32_t stride0, std::uint32_t stride1,
+                          Tensor &y) override;
+  void max_pool2d_bw_impl(const Tensor &x, const Tensor &y, const Tensor &gy, std::uint32_t window0,
+                          std::uint32_t window1, std::uint32_t padding0, std::uint32_t padding1,
+                          std::uint32_t stride0, std::uint32_t stride1, Tensor &gx) override;
 
   // Bytes of device storage for `n` elements (16-bit storage rounds the
   // element count up to even, as devices::CUDA16 does).
