@@ -1,7 +1,7 @@
 #ifndef PRIMITIV_DEVICES_HIP_DEVICE_H_
 #define PRIMITIV_DEVICES_HIP_DEVICE_H_
 
-// primitiv::devices::HIP -- AMD MI355X (gfx950) backend for the matmul path.
+// primitiv::devices::HIP -- AMD MI355X (gfx950) backend.
 //
 // Drop-in subclass of primitiv::Device (primitiv/core/device.h): the existing
 // Graph / Node / Tensor / Parameter code talks to it through the same virtual
@@ -9,11 +9,11 @@
 // work goes through libphip's C ABI (phip.h); this class only owns the
 // context and the memory pool and forwards each operation.
 //
-// Implemented: matmul forward/backward and the helpers the graph needs around
-// them (allocation, fill, host<->device and device<->device copies, in-place
-// add with minibatch broadcasting, minibatch sum).  Every other operation
-// throws primitiv::NotImplementedError, as the reference's own backends do for
-// operations they lack (primitiv/devices/opencl/ops/conv2d.cc:16,25).
+// Every operation of the Device interface is implemented: matmul
+// forward/backward (the path this backend was built around), the helpers the
+// graph needs around them (allocation, fill, copies, in-place add with
+// minibatch broadcasting, minibatch sum), the elementwise families, indexing
+// and reductions, random tensors, convolution and pooling.
 
 #include <cstdint>
 #include <memory>
