@@ -107,13 +107,6 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const T *gcol, T *gx, co
   *dst = from_f32<T>(to_f32(*dst) + sum);
 }
 
-inline unsigned blocks_for(long total, int cus) {
-  long b = (total + kBlock - 1) / kBlock;
-  const long cap = (long)cus * 16;
-  if (b > cap) b = cap;
-  return (unsigned)(b < 1 ? 1 : b);
-}
-
 template <typename T>
 int run_gemm(phip_ctx *ctx, const Gemm &p) {
   if constexpr (sizeof(T) == 4) return gemm_f32(ctx, p);
@@ -351,11 +344,12 @@ struct PoolGeom {
 };
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void max_pool2d_fw_kernel(const T *x, T *y, const PoolGeom g, long total) {
+__global__ __launch_bounds__(kBlock) void max_pool2d_fw_kernel(const T *x, T *y, const PoolGeom g) {
   const long plane_y = (long)g.OH * g.OW, plane_x = (long)g.H * g.W;
-  for (long i = (long)blockIdx.x * kBlock + threadIdx.x; i < total; i += (long)gridDim.x * kBlock) {
-    const long r = i / plane_y;
-    const int n = (int)(i - r * plane_y);
+  const int n = blockIdx.x * kBlock + threadIdx.x;
+  if (n < plane_y) {
+    const long r = blockIdx.y + (long)blockIdx.z * gridDim.y;
+    const long i = r * plane_y + n;
     const int ox = n / g.OH, oy = n - ox * g.OH;
     const T *xs = x + r * plane_x;
     float best = -3.402823466e+38f;  // the lowest finite float, as std::numeric_limits<float>::lowest()
@@ -376,11 +370,12 @@ __global__ __launch_bounds__(kBlock) void max_pool2d_fw_kernel(const T *x, T *y,
 // position (inside x's plane) of the first element of each window equal to y
 template <typename T>
 __global__ __launch_bounds__(kBlock) void max_pool2d_where_kernel(const T *x, const T *y, uint32_t *where,
-                                                                 const PoolGeom g, long total) {
+                                                                 const PoolGeom g) {
   const long plane_y = (long)g.OH * g.OW, plane_x = (long)g.H * g.W;
-  for (long i = (long)blockIdx.x * kBlock + threadIdx.x; i < total; i += (long)gridDim.x * kBlock) {
-    const long r = i / plane_y;
-    const int n = (int)(i - r * plane_y);
+  const int n = blockIdx.x * kBlock + threadIdx.x;
+  if (n < plane_y) {
+    const long r = blockIdx.y + (long)blockIdx.z * gridDim.y;
+    const long i = r * plane_y + n;
     const int ox = n / g.OH, oy = n - ox * g.OH;
     const T *xs = x + r * plane_x;
     const float target = to_f32(y[i]);
@@ -403,11 +398,12 @@ __global__ __launch_bounds__(kBlock) void max_pool2d_where_kernel(const T *x, co
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void max_pool2d_bw_kernel(const T *gy, const uint32_t *where, T *gx,
-                                                              const PoolGeom g, long total) {
+                                                              const PoolGeom g) {
   const long plane_y = (long)g.OH * g.OW, plane_x = (long)g.H * g.W;
-  for (long i = (long)blockIdx.x * kBlock + threadIdx.x; i < total; i += (long)gridDim.x * kBlock) {
-    const long r = i / plane_x;
-    const int p = (int)(i - r * plane_x);
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p < plane_x) {
+    const long r = blockIdx.y + (long)blockIdx.z * gridDim.y;
+    const long i = r * plane_x + p;
     const int xx = p / g.H, xy = p - xx * g.H;
     // windows (oy, ox) that contain (xy, xx): o*str - pad <= x < o*str - pad + win
     const int ty = xy + g.pad0, tx = xx + g.pad1;
@@ -428,6 +424,53 @@ __global__ __launch_bounds__(kBlock) void max_pool2d_bw_kernel(const T *gy, cons
       }
     if (any) gx[i] = from_f32<T>(to_f32(gx[i]) + sum);
   }
+}
+
+// Windows that do not overlap (stride >= window on both axes): every element of
+// gx belongs to at most one window, so the thread that owns an output finds the
+// first element equal to y and adds gy to it directly - one launch, no scratch.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void max_pool2d_bw_disjoint_kernel(const T *x, const T *y, const T *gy, T *gx,
+                                                                       const PoolGeom g) {
+  const int plane_y = g.OH * g.OW;
+  const int n = blockIdx.x * kBlock + threadIdx.x;
+  if (n >= plane_y) return;
+  const long r = blockIdx.y + (long)blockIdx.z * gridDim.y;
+  const long plane_x = (long)g.H * g.W;
+  const int ox = n / g.OH, oy = n - ox * g.OH;
+  const T *xs = x + r * plane_x;
+  const float target = to_f32(y[r * plane_y + n]);
+  for (int wx = 0; wx < g.win1; ++wx) {
+    const int xx = ox * g.str1 - g.pad1 + wx;
+    if (xx < 0 || xx >= g.W) continue;
+    for (int wy = 0; wy < g.win0; ++wy) {
+      const int xy = oy * g.str0 - g.pad0 + wy;
+      if (xy < 0 || xy >= g.H) continue;
+      const long p = (long)xx * g.H + xy;
+      if (to_f32(xs[p]) == target) {
+        T *dst = gx + r * plane_x + p;
+        *dst = from_f32<T>(to_f32(*dst) + to_f32(gy[r * plane_y + n]));
+        return;
+      }
+    }
+  }
+}
+
+// Calls launch(first_plane, grid_y, grid_z) until `repeat` planes are covered;
+// a kernel finds its plane as first_plane + blockIdx.y + blockIdx.z * gridDim.y.
+template <typename F>
+int for_plane_grids(uint32_t repeat, F launch) {
+  const unsigned wide = repeat < 65535u ? repeat : 65535u;
+  for (uint32_t r0 = 0; r0 < repeat;) {
+    const uint32_t left = repeat - r0;
+    unsigned gz = left / wide;
+    if (gz > 65535u) gz = 65535u;
+    const unsigned yd = gz == 0 ? left : wide, zd = gz == 0 ? 1u : gz;
+    launch(r0, yd, zd);
+    PHIP_LAUNCH_CHECK();
+    r0 += yd * zd;
+  }
+  return PHIP_OK;
 }
 
 struct PoolArgs {
@@ -458,11 +501,11 @@ int max_pool2d_fw(phip_ctx *ctx, const void *x, void *y, const PoolArgs &a) {
   PoolGeom g;
   const int rc = pool_geometry(a, &g);
   if (rc != PHIP_OK) return rc;
-  const long total = (long)g.OH * g.OW * a.repeat;
-  hipLaunchKernelGGL(max_pool2d_fw_kernel<T>, dim3(blocks_for(total, ctx->prop.multiProcessorCount)), dim3(kBlock), 0,
-                     ctx->stream, static_cast<const T *>(x), static_cast<T *>(y), g, total);
-  PHIP_LAUNCH_CHECK();
-  return PHIP_OK;
+  const long px = (long)g.H * g.W, py = (long)g.OH * g.OW;
+  return for_plane_grids(a.repeat, [&](uint32_t r0, unsigned yd, unsigned zd) {
+    hipLaunchKernelGGL(max_pool2d_fw_kernel<T>, dim3((unsigned)((py + kBlock - 1) / kBlock), yd, zd), dim3(kBlock), 0,
+                       ctx->stream, static_cast<const T *>(x) + r0 * px, static_cast<T *>(y) + r0 * py, g);
+  });
 }
 
 template <typename T>
@@ -473,19 +516,30 @@ int max_pool2d_bw(phip_ctx *ctx, const void *x, const void *y, const void *gy, v
   PoolGeom g;
   int rc = pool_geometry(a, &g);
   if (rc != PHIP_OK) return rc;
-  const int cus = ctx->prop.multiProcessorCount;
-  const long outputs = (long)g.OH * g.OW * a.repeat, inputs = (long)g.H * g.W * a.repeat;
+  const long px = (long)g.H * g.W, py = (long)g.OH * g.OW;
+  const T *xp = static_cast<const T *>(x), *yp = static_cast<const T *>(y), *gyp = static_cast<const T *>(gy);
+  T *gxp = static_cast<T *>(gx);
+  if (g.str0 >= g.win0 && g.str1 >= g.win1) {
+    return for_plane_grids(a.repeat, [&](uint32_t r0, unsigned yd, unsigned zd) {
+      hipLaunchKernelGGL(max_pool2d_bw_disjoint_kernel<T>, dim3((unsigned)((py + kBlock - 1) / kBlock), yd, zd),
+                         dim3(kBlock), 0, ctx->stream, xp + r0 * px, yp + r0 * py, gyp + r0 * py, gxp + r0 * px, g);
+    });
+  }
   void *block = nullptr;
-  rc = phip_pool_alloc(ctx, sizeof(uint32_t) * (size_t)outputs, &block, nullptr);
+  rc = phip_pool_alloc(ctx, sizeof(uint32_t) * (size_t)py * a.repeat, &block, nullptr);
   if (rc != PHIP_OK) return rc;
   uint32_t *where = static_cast<uint32_t *>(block);
-  hipLaunchKernelGGL(max_pool2d_where_kernel<T>, dim3(blocks_for(outputs, cus)), dim3(kBlock), 0, ctx->stream,
-                     static_cast<const T *>(x), static_cast<const T *>(y), where, g, outputs);
-  hipLaunchKernelGGL(max_pool2d_bw_kernel<T>, dim3(blocks_for(inputs, cus)), dim3(kBlock), 0, ctx->stream,
-                     static_cast<const T *>(gy), where, static_cast<T *>(gx), g, inputs);
+  rc = for_plane_grids(a.repeat, [&](uint32_t r0, unsigned yd, unsigned zd) {
+    hipLaunchKernelGGL(max_pool2d_where_kernel<T>, dim3((unsigned)((py + kBlock - 1) / kBlock), yd, zd), dim3(kBlock),
+                       0, ctx->stream, xp + r0 * px, yp + r0 * py, where + r0 * py, g);
+  });
+  if (rc == PHIP_OK)
+    rc = for_plane_grids(a.repeat, [&](uint32_t r0, unsigned yd, unsigned zd) {
+      hipLaunchKernelGGL(max_pool2d_bw_kernel<T>, dim3((unsigned)((px + kBlock - 1) / kBlock), yd, zd), dim3(kBlock), 0,
+                         ctx->stream, gyp + r0 * py, where + r0 * py, gxp + r0 * px, g);
+    });
   phip_pool_free(ctx, block);  // the stream is in order: reusable behind these launches
-  PHIP_LAUNCH_CHECK();
-  return PHIP_OK;
+  return rc;
 }
 
 }  // namespace

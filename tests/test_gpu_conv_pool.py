@@ -168,6 +168,8 @@ POOL_RANDOM = [  # x dims, batch, (win0, win1, pad0, pad1, str0, str1)
     ([9, 31, 4], 1, (9, 31, 0, 0, 1, 1)),       # one window per plane
     ([12, 10, 2], 4, (3, 2, 2, 1, 1, 3)),
     ([64, 64], 2, (5, 5, 2, 2, 1, 1)),
+    ([17, 13, 3], 2, (2, 3, 1, 2, 2, 3)),       # disjoint windows with padding
+    ([20, 21, 2], 3, (2, 2, 1, 1, 3, 4)),       # gaps between the windows
 ]
 
 
