@@ -105,3 +105,81 @@ def test_matmul_gradients_of_one_tensor_used_twice(dev):
     want = (G @ A.T + A.T @ G).T.reshape(-1)
     tol = 1e-4 if dev._SUFFIX == "f32" else 2e-2
     assert np.max(np.abs(g.to_vector() - want)) <= tol * np.max(np.abs(want))
+
+
+def test_small_convolutional_network_against_oracle(dev):
+    # conv 3x3 -> relu -> 2x2 max pooling, twice, then a dense layer: the layer sequence of the
+    # reference's examples/mnist/mnist_cnn (smaller), forward and backward, every node compared
+    # with the CPU oracle fed the same values
+    import oracle
+    from util import norm_rel_err
+    tol = 1e-4 if dev._SUFFIX == "f32" else 3e-2
+    rng = np.random.default_rng(11)
+    bs = 4
+    x = rng.standard_normal(12 * 12 * bs).astype(np.float32)
+    w1 = (0.4 * rng.standard_normal(3 * 3 * 1 * 4)).astype(np.float32)
+    w2 = (0.3 * rng.standard_normal(3 * 3 * 4 * 8)).astype(np.float32)
+    w3 = (0.2 * rng.standard_normal(10 * 72)).astype(np.float32)
+    conv, pool = (1, 1, 1, 1, 1, 1), (2, 2, 0, 0, 2, 2)
+    tx = dev.new_tensor_by_vector(S([12, 12, 1], bs), x)
+    tw1 = dev.new_tensor_by_vector(S([3, 3, 1, 4]), w1)
+    tw2 = dev.new_tensor_by_vector(S([3, 3, 4, 8]), w2)
+    tw3 = dev.new_tensor_by_vector(S([10, 72]), w3)
+
+    # forward on the device
+    c1 = dev.conv2d_fw(tx, tw1, *conv)
+    r1 = dev.const_fw("prelu", c1, 0.0)
+    p1 = dev.max_pool2d_fw(r1, *pool)
+    c2 = dev.conv2d_fw(p1, tw2, *conv)
+    r2 = dev.const_fw("prelu", c2, 0.0)
+    p2 = dev.max_pool2d_fw(r2, *pool)
+    assert p2.shape() == S([3, 3, 8], bs)
+    flat = dev.new_tensor_by_vector(S([72], bs), p2.to_vector())      # flatten: same memory order
+    out = dev.matmul_fw(tw3, flat)
+
+    # the same on the oracle, each layer fed the DEVICE's input of that layer so that
+    # 16-bit rounding does not pile up across layers
+    def near(t, want, what):
+        assert norm_rel_err(t.to_vector(), want) <= tol, what
+
+    near(c1, oracle.conv2d_fw(x, w1, [12, 12, 1], bs, [3, 3, 1, 4], 1, *conv), "conv1")
+    near(r1, oracle.const_fw("prelu", c1.to_vector(), 0.0), "relu1")
+    near(p1, oracle.max_pool2d_fw(r1.to_vector(), [12, 12, 4], bs, *pool), "pool1")
+    near(c2, oracle.conv2d_fw(p1.to_vector(), w2, [6, 6, 4], bs, [3, 3, 4, 8], 1, *conv), "conv2")
+    near(p2, oracle.max_pool2d_fw(r2.to_vector(), [6, 6, 8], bs, *pool), "pool2")
+    near(out, oracle.matmul_fw(w3, flat.to_vector(), 10, 72, 1, 1, bs), "dense")
+
+    # backward from d(out) = 1, gradients starting at zero
+    zeros = lambda like: dev.new_tensor_by_constant(like.shape(), 0)
+    g_out = dev.new_tensor_by_constant(out.shape(), 1)
+    g_w3, g_flat = zeros(tw3), zeros(flat)
+    dev.matmul_bw(tw3, flat, out, g_out, g_w3, g_flat)
+    g_p2 = dev.new_tensor_by_vector(p2.shape(), g_flat.to_vector())
+    g_r2 = zeros(r2)
+    dev.max_pool2d_bw(r2, p2, g_p2, *pool, g_r2)
+    g_c2 = zeros(c2)
+    dev.const_bw("prelu", c2, r2, g_r2, 0.0, g_c2)
+    g_p1, g_w2 = zeros(p1), zeros(tw2)
+    dev.conv2d_bw(p1, tw2, c2, g_c2, *conv, g_p1, g_w2)
+    g_r1 = zeros(r1)
+    dev.max_pool2d_bw(r1, p1, g_p1, *pool, g_r1)
+    g_c1 = zeros(c1)
+    dev.const_bw("prelu", c1, r1, g_r1, 0.0, g_c1)
+    g_x, g_w1 = zeros(tx), zeros(tw1)
+    dev.conv2d_bw(tx, tw1, c1, g_c1, *conv, g_x, g_w1)
+
+    z = lambda n: np.zeros(n, np.float32)
+    ones = np.ones(10 * bs, np.float32)
+    rg_w3, rg_flat = oracle.matmul_bw(w3, flat.to_vector(), ones, z(720), z(72 * bs), 10, 72, 1, 1, bs)
+    near(g_w3, rg_w3, "g_w3")
+    near(g_flat, rg_flat, "g_flat")
+    near(g_r2, oracle.max_pool2d_bw(r2.to_vector(), p2.to_vector(), g_p2.to_vector(), z(6 * 6 * 8 * bs), [6, 6, 8], bs,
+                                    *pool), "g_r2")
+    near(g_c2, oracle.const_bw("prelu", c2.to_vector(), r2.to_vector(), g_r2.to_vector(), 0.0, z(6 * 6 * 8 * bs)), "g_c2")
+    rg_p1, rg_w2 = oracle.conv2d_bw(p1.to_vector(), w2, g_c2.to_vector(), z(6 * 6 * 4 * bs), z(w2.size), [6, 6, 4], bs,
+                                    [3, 3, 4, 8], 1, *conv)
+    near(g_p1, rg_p1, "g_p1")
+    near(g_w2, rg_w2, "g_w2")
+    rg_x, rg_w1 = oracle.conv2d_bw(x, w1, g_c1.to_vector(), z(x.size), z(w1.size), [12, 12, 1], bs, [3, 3, 1, 4], 1, *conv)
+    near(g_x, rg_x, "g_x")
+    near(g_w1, rg_w1, "g_w1")
