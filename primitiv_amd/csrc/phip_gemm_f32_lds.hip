@@ -6,6 +6,11 @@
 // v_mfma_f32_32x32x2_f32 tiles.  Two 32 KiB LDS stages (A region then B region,
 // 16 KiB each); two workgroups share a CU.
 //
+// SPLIT: a problem with too few output tiles for the chip cuts its K range
+// between workgroups; an accumulating product adds its tiles into C with fp32
+// atomics, an overwriting one meets through partial tiles and a per-tile
+// ticket (see last_of_tile).  The unsplit instantiation carries none of that.
+//
 // The LDS image of an operand tile is described with the loader that builds it.
 #include "phip_gemm_f32_lds.h"
 
@@ -17,7 +22,7 @@ constexpr int kRegion = 16384;            // bytes per operand per stage
 constexpr int kStage = 2 * kRegion;
 constexpr int kLdsBytes = 2 * kStage;
 
-template <bool A_KMAJOR, bool B_KMAJOR>
+template <bool A_KMAJOR, bool B_KMAJOR, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs d) {
   const GemmArgs &g = d.g;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
@@ -30,6 +35,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
   int t = xcd_remap(blockIdx.x, gridDim.x);
   const int tile_m = t % g.tiles_m; t /= g.tiles_m;
   const int tile_n = t % g.tiles_n; t /= g.tiles_n;
+  int split = 0;
+  if constexpr (SPLIT) {
+    split = t % g.splits;
+    t /= g.splits;
+  }
   const int z = t;
   const int m0 = tile_m * LBM, n0 = tile_n * LBN;
 
@@ -53,12 +63,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  const int kt_end = g.total_ktiles;
+  // K tiles [kt_base, kt_base + kt_end) belong to this workgroup
+  const int kt_base = SPLIT ? (int)((long)split * g.total_ktiles / g.splits) : 0;
+  const int kt_end = SPLIT ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
   auto issue_tile = [&](int kt, int q) {
     // instruction q of the 8 that move K tile kt (4 for A, then 4 for B)
     const bool live = kt < kt_end;
-    const int ktc = live ? kt : 0;
+    const int ktc = live ? kt + kt_base : 0;
     const int r = ktc / g.ktiles_per_r;
     const int kt_in_r = ktc - r * g.ktiles_per_r;
     const uint32_t stage = lds_base + (uint32_t)(kt & 1) * kStage;
@@ -113,25 +125,52 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
 
   float *Cz = g.C + (long)z * g.sC;
   const bool interior = m0 + LBM <= g.M && n0 + LBN <= g.N;
+  int ns[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) ns[v] = 8 * (v / 4) + (v % 4);
+  if constexpr (SPLIT) {
+    if (g.atomic == 2) {
+      // leave the partial tile; the last workgroup of the output tile adds the ranges in order
+      __shared__ uint32_t last_flag;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float vals[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) vals[v] = acc[i][j][v];
+          store_partial<16>(g, z, split, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, ns, vals);
+        }
+      if (!last_of_tile(g, (z * g.tiles_n + tile_n) * g.tiles_m + tile_m, &last_flag)) return;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float vals[16];
+          sum_partials<16>(g, z, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, ns, vals);
+          emit_c<16>(Cz, g.ldc, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, g.M, g.N, interior, ns, vals, 0,
+                     g.accumulate);
+        }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       float vals[16];
-      int ns[16];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        vals[v] = acc[i][j][v];
-        ns[v] = 8 * (v / 4) + (v % 4);
-      }
-      emit_c<16>(Cz, g.ldc, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, g.M, g.N, interior, ns, vals, 0,
-                 g.accumulate);
+      for (int v = 0; v < 16; ++v) vals[v] = acc[i][j][v];
+      emit_c<16>(Cz, g.ldc, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, g.M, g.N, interior, ns, vals,
+                 SPLIT ? g.atomic : 0, g.accumulate);
     }
 }
 
 }  // namespace
 
-// Large, 16-byte-aligned problems.  Sets *handled when it launched.
+// Large, 16-byte-aligned problems: at least one 128 x 128 tile per CU, or an
+// eighth of that with a K long enough to be cut between workgroups.  Sets
+// *handled when it launched.
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
   auto aligned = [](const void *ptr, long ld, long s, long r) {
@@ -144,8 +183,29 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   if (a_bytes >= (1L << 31) || b_bytes >= (1L << 31)) return PHIP_OK;
   const long tiles = (long)((p.M + LBM - 1) / LBM) * ((p.N + LBN - 1) / LBN) * p.batch;
   const int cus = ctx->prop.multiProcessorCount;
-  if (tiles < cus || (long)p.K * p.rbatch <= 128 || tiles > 0x7fffffffL) return PHIP_OK;
+  if ((long)p.K * p.rbatch <= 128 || tiles > 0x7fffffffL) return PHIP_OK;
   if (p.a_kmajor && !p.b_kmajor) return PHIP_OK;
+  const long total_ktiles = (long)((p.K + LBK - 1) / LBK) * p.rbatch;
+  // Fewer tiles than CUs: worth it for a long K (from 2048) cut into ranges of at least 8 K tiles, when the
+  // tiles alone fill between an eighth and three quarters of the CUs (measured on M, N in 512 .. 4096: with
+  // a shorter K, or more tiles, the staged 64 x 64 tiles are as fast or faster).  The number of ranges
+  // minimises a small cost model fitted to those measurements: a fixed cost per workgroup, the time of a K
+  // tile when a workgroup has its CU to itself or shares it with a second one, and the exchange of the
+  // partial results, which grows with the number of ranges.
+  long splits = 1;
+  if (tiles < cus) {
+    if (total_ktiles < 64 || tiles * 8 < cus || tiles * 4 >= cus * 3L) return PHIP_OK;
+    double best = 0.0;
+    for (long s = 2; s <= 16 && s * 8 <= total_ktiles && tiles * s <= 2L * cus; ++s) {
+      const double per_ktile = tiles * s <= cus ? 2.6 : 4.2;  // microseconds
+      const double t = 8.0 + per_ktile * (double)total_ktiles / (double)s + 3.0 * (double)s;
+      if (splits == 1 || t < best) {
+        best = t;
+        splits = s;
+      }
+    }
+    if (splits < 2) return PHIP_OK;
+  }
 
   LdsArgs d;
   GemmArgs &a = d.g;
@@ -158,27 +218,54 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   a.rA = p.rA; a.rB = p.rB;
   a.tiles_m = (p.M + LBM - 1) / LBM;
   a.tiles_n = (p.N + LBN - 1) / LBN;
-  a.splits = 1;
+  a.splits = (int)splits;
   a.ktiles_per_r = (p.K + LBK - 1) / LBK;
-  a.total_ktiles = a.ktiles_per_r * p.rbatch;
-  a.atomic = 0;
+  a.total_ktiles = (int)total_ktiles;
+  a.atomic = splits > 1;
   a.accumulate = p.accumulate ? 1 : 0;
   a.partial = nullptr;
-  a.tickets = nullptr;
+  a.tickets = ctx->tile_tickets;
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
 
-#define PHIP_LDS(SLOT, AK, BKM)                                                                 \
-  do {                                                                                          \
-    auto kern = gemm_f32_lds_kernel<AK, BKM>;                                                   \
-    const int rc = raise_lds_limit(ctx, SLOT, reinterpret_cast<const void *>(kern), kLdsBytes); \
-    if (rc != PHIP_OK) return rc;                                                               \
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), kLdsBytes, ctx->stream, d); \
+  // A split overwriting product: fp32 partial tiles in scratch memory, summed by the last workgroup of
+  // each tile; without room for them, a zero fill and atomics.
+  void *block = nullptr;
+  if (splits > 1 && !p.accumulate) {
+    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
+    if (tiles <= kTicketSlots && bytes <= (size_t)(256L << 20) && phip_pool_alloc(ctx, bytes, &block, nullptr) == PHIP_OK) {
+      a.atomic = 2;
+      a.partial = static_cast<float *>(block);
+    } else {
+      const long total = (long)p.M * p.N * p.batch;
+      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+      if (blocks > cus * 8L) blocks = cus * 8L;
+      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N,
+                         p.ldc, p.sC, p.batch);
+      PHIP_LAUNCH_CHECK();
+    }
+  }
+
+  int rc = PHIP_OK;
+#define PHIP_LDS(SLOT, AK, BKM, SP)                                                                          \
+  do {                                                                                                       \
+    auto kern = gemm_f32_lds_kernel<AK, BKM, SP>;                                                            \
+    rc = raise_lds_limit(ctx, SLOT + (SP ? 3 : 0), reinterpret_cast<const void *>(kern), kLdsBytes);         \
+    if (rc == PHIP_OK)                                                                                       \
+      hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * splits)), dim3(kThreads), kLdsBytes, ctx->stream, d); \
   } while (0)
-  if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true);
-  else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false);
-  else PHIP_LDS(kSlotGemmF32Lds + 2, true, true);
+  if (splits > 1) {
+    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, true);
+    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, true);
+    else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, true);
+  } else {
+    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, false);
+    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, false);
+    else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, false);
+  }
 #undef PHIP_LDS
+  if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
+  if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
   *handled = true;
   return PHIP_OK;

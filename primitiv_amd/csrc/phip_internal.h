@@ -80,7 +80,7 @@ constexpr int kTicketSlots = 65536;
 // Bits of phip_ctx::lds_limit_raised: first slot of each kernel family that
 // asks for a dynamic LDS size (one slot per instantiation, counted from here).
 enum LdsSlot {
-  kSlotGemmF32Lds = 0,    // 3 instantiations
+  kSlotGemmF32Lds = 0,    // 6 instantiations
   kSlotGemmH16Big = 8,    // 6
   kSlotGemmF32Slab = 16,  // 5
   kSlotGemmF32RankK = 21, // 2

@@ -300,11 +300,41 @@ def test_gradients_into_one_buffer(dev):
     assert norm_rel_err(tg.to_vector(), rga + rgb) <= F32_TOL
 
 
+# mid-size products with a long K (from 2048) and fewer 128 x 128 tiles than CUs: the large-tile
+# kernel with its K range cut between workgroups - forward (partial tiles and tickets), both
+# gradients (atomics), ragged edges, per-sample products, a contraction over the minibatch
+MIDSIZE_F32 = [  # di, dj, dk, ba, bb
+    (1536, 2048, 512, 1, 1),
+    (1024, 1024, 2048, 1, 1),
+    (2048, 1024, 1024, 1, 1),
+    (1028, 1100, 2052, 1, 1),
+    (520, 2080, 300, 3, 3),
+    (700, 1040, 520, 3, 1),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", MIDSIZE_F32)
+def test_midsize_long_k_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di + 2 * dj + 3 * dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    y, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(y, ry) <= F32_TOL
+    assert norm_rel_err(ga, rga) <= F32_TOL
+    assert norm_rel_err(gb, rgb) <= F32_TOL
+
+
 # an overwriting product with few output tiles and a long K is cut between workgroups
 # that meet through partial tiles, summed in a fixed order by whichever finishes last:
 # right, and the same bits on every run
 @pytest.mark.parametrize("di,dj,dk,ba,bb", [(256, 784, 1, 1, 128), (64, 3000, 1, 1, 40), (100, 5000, 33, 1, 1),
-                                            (48, 2048, 8, 3, 3)])
+                                            (48, 2048, 8, 3, 3), (1028, 2052, 1100, 1, 1)])
 def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
     rng = np.random.default_rng(di + dj)
     a = rng.standard_normal(di * dj * ba).astype(np.float32)
