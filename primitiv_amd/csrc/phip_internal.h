@@ -84,6 +84,7 @@ enum LdsSlot {
   kSlotGemmH16Big = 8,    // 6
   kSlotGemmF32Slab = 16,  // 5
   kSlotGemmF32RankK = 21, // 2
+  kSlotGemmH16Mid = 23,   // 6
 };
 
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on
