@@ -11,6 +11,7 @@ workload (square batched fp32), `workloads` carries the same figures for all
 five.  The CPU figures come from the CPU oracle timed on this host.
 """
 import argparse
+import copy
 import ctypes
 import json
 import os
@@ -98,7 +99,7 @@ def cpu_baseline(w, threads=1):
     of the workload and scales to TFLOP/s."""
     import oracle
     steps, bb, repeats, sample = w.steps, w.bb, 2, "full workload"
-    if w.name == "half_storage":
+    if w.name.startswith("half_storage"):
         bb, repeats, sample = 1, 1, "1 of the 8 minibatch samples (a shared), fp32"
     elif w.name == "square_batched":
         sample = "one fw+bw call, all 16 samples"
@@ -122,8 +123,18 @@ def cpu_baseline(w, threads=1):
             "sample": "%s, best of %d, %.2f s" % (sample, repeats, best)}
 
 
+def _workload(name):
+    """A workload of the table, or its half-storage entry with bfloat16 storage (same shapes, same
+    inputs; not one of the reference's configurations, reported next to them)."""
+    if name == "half_storage_bf16":
+        w = copy.copy(WORKLOADS["half_storage"])
+        w.name, w.storage = name, "bf16"
+        return w
+    return WORKLOADS[name]
+
+
 def measure(name, steps, warmup, skip_cpu):
-    w = WORKLOADS[name]
+    w = _workload(name)
     dev = pa.HIP(0) if w.storage == "f32" else pa.HIP16(0, storage=w.storage)
     res = Resident(dev, w)
     host_s, ev_s = time_gpu(dev, res, steps, warmup)
@@ -342,7 +353,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", help="all or one of: " + ", ".join(WORKLOADS))
+    ap.add_argument("--workload", default="all",
+                    help="all or one of: " + ", ".join(list(WORKLOADS) + ["half_storage_bf16"]))
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one streaming y += x over 64 Mi floats (reads 512 MiB, writes 256 MiB): "
@@ -374,13 +386,14 @@ def main():
         del x, y
         dev.close()
 
-    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    names = list(WORKLOADS) + ["half_storage_bf16"] if args.workload == "all" else [args.workload]
     if HEADLINE not in names and args.workload == "all":
         names.append(HEADLINE)
     results = {}
     for n in names:
-        steps = args.steps if n != "half_storage" else max(1, min(args.steps, 5))
-        results[n] = measure(n, steps, args.warmup, args.skip_cpu)
+        steps = args.steps if not n.startswith("half_storage") else max(1, min(args.steps, 5))
+        # the CPU figure of the bf16 variant would repeat the fp16 one: same shapes, fp32 on the CPU
+        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16")
         print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)"
               % (n, results[n]["ms_per_step"], results[n]["tflops"], 100 * results[n]["frac_mfma_peak"],
                  results[n]["gbs"], 100 * results[n]["frac_hbm_peak"]), file=sys.stderr, flush=True)

@@ -81,6 +81,19 @@ __device__ inline uint32_t round_c(float x) {
   else return __builtin_bit_cast(uint16_t, from_f32<f16_t>(x));
 }
 
+// Two results rounded to nearest even and packed, x0 in the low half.  bf16 has
+// an instruction for exactly that (NaNs stay NaNs); fp16 converts one by one.
+template <bool BF16>
+__device__ inline uint32_t round_pair(float x0, float x1) {
+  if constexpr (BF16) {
+    uint32_t r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(x0), "v"(x1));
+    return r;
+  } else {
+    return round_c<false>(x0) | (round_c<false>(x1) << 16);
+  }
+}
+
 // Writes the 128 x 128 block of results one wavefront holds into the 16-bit C,
 // 16 bytes (8 consecutive rows of one column) per lane and store instruction.
 // The matrix instruction leaves a lane with one row and 16 columns of each
@@ -159,7 +172,7 @@ __device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, i
           x0 += widen<BF16>(old[it][e] & 0xffffu);
           x1 += widen<BF16>(old[it][e] >> 16);
         }
-        out[e] = round_c<BF16>(x0) | (round_c<BF16>(x1) << 16);
+        out[e] = round_pair<BF16>(x0, x1);
       }
       if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(4 * it) * ldc) = out;
     }
@@ -227,7 +240,7 @@ __device__ inline void emit_block64_via_lds(float *area, uint16_t *Cz, long ldc,
         x0 += widen<BF16>(old[it][e] & 0xffffu);
         x1 += widen<BF16>(old[it][e] >> 16);
       }
-      out[e] = round_c<BF16>(x0) | (round_c<BF16>(x1) << 16);
+      out[e] = round_pair<BF16>(x0, x1);
     }
     if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(8 * it) * ldc) = out;
   }
