@@ -75,23 +75,14 @@ __device__ inline float widen(uint32_t bits16) {
   else return to_f32(__builtin_bit_cast(f16_t, (uint16_t)bits16));
 }
 
-template <bool BF16>
-__device__ inline uint32_t round_c(float x) {
-  if constexpr (BF16) return from_f32<bf16_t>(x).bits;
-  else return __builtin_bit_cast(uint16_t, from_f32<f16_t>(x));
-}
-
-// Two results rounded to nearest even and packed, x0 in the low half.  bf16 has
-// an instruction for exactly that (NaNs stay NaNs); fp16 converts one by one.
+// Two results rounded to nearest even (the mode these conversions run in by
+// default) and packed, x0 in the low half: one instruction per pair.
 template <bool BF16>
 __device__ inline uint32_t round_pair(float x0, float x1) {
-  if constexpr (BF16) {
-    uint32_t r;
-    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(x0), "v"(x1));
-    return r;
-  } else {
-    return round_c<false>(x0) | (round_c<false>(x1) << 16);
-  }
+  uint32_t r;
+  if constexpr (BF16) asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(x0), "v"(x1));
+  else asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(x0), "v"(x1));
+  return r;
 }
 
 // Writes the 128 x 128 block of results one wavefront holds into the 16-bit C,
