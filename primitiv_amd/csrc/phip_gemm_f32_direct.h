@@ -260,13 +260,14 @@ inline bool plan_direct(const phip_ctx *ctx, const Gemm &p, DirectPlan *plan) {
   // Split K between workgroups until about two workgroups per CU are busy,
   // keeping at least 4 chunks (32 k) per wavefront (measured best on the
   // recurrent-gate and output-projection gradients).  An overwriting product
-  // is only split when it would otherwise leave most of the chip idle: its
-  // ranges meet through partial tiles in scratch memory.
+  // is only split when it would otherwise leave most of the chip idle, or when
+  // K is long (from 2048) and the tiles are fewer than the CUs: its ranges meet
+  // through partial tiles in scratch memory.
   int splits = 1;
   const long want = (2L * cus + t - 1) / t;
   long cap = d.total_chunks / 16;
   if (cap < 1) cap = 1;
-  if (p.accumulate || t * 8 <= cus) splits = (int)(want < cap ? want : cap);
+  if (p.accumulate || t * 8 <= cus || (d.total_chunks >= 256 && t < cus)) splits = (int)(want < cap ? want : cap);
   if (splits < 1) splits = 1;
   // An overwriting product whose K fits one round of loads of 8 wavefronts (at
   // most 8 chunks each) takes 8 wavefronts per workgroup.  (16 wavefronts for a
