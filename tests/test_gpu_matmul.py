@@ -334,7 +334,8 @@ def test_midsize_long_k_f32(dev, di, dj, dk, ba, bb):
 # that meet through partial tiles, summed in a fixed order by whichever finishes last:
 # right, and the same bits on every run
 @pytest.mark.parametrize("di,dj,dk,ba,bb", [(256, 784, 1, 1, 128), (64, 3000, 1, 1, 40), (100, 5000, 33, 1, 1),
-                                            (48, 2048, 8, 3, 3), (1028, 2052, 1100, 1, 1)])
+                                            (48, 2048, 8, 3, 3), (1028, 2052, 1100, 1, 1),
+                                            (1024, 4096, 1, 1, 128)])
 def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
     rng = np.random.default_rng(di + dj)
     a = rng.standard_normal(di * dj * ba).astype(np.float32)
