@@ -166,11 +166,182 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
     }
 }
 
+// The same scheme with 64 x 64 x 32 tiles for problems with too few 128 x 128
+// tiles: 2 x 2 wavefronts of one 32 x 32 block each (16 accumulator registers),
+// two 16 KiB stages, four workgroups per CU, so that the matrix pipe of a SIMD
+// has four wavefronts to draw from while any of them waits at a barrier.
+constexpr int SBM = 64, SBN = 64;
+constexpr int kRegion64 = 8192;
+constexpr int kStage64 = 2 * kRegion64;
+constexpr int kLds64Bytes = 2 * kStage64;
+
+template <bool A_KMAJOR, bool B_KMAJOR, bool SPLIT>
+__global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsArgs d) {
+  const GemmArgs &g = d.g;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+
+  int t = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
+  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
+  int split = 0;
+  if constexpr (SPLIT) {
+    split = t % g.splits;
+    t /= g.splits;
+  }
+  const int z = t;
+  const int m0 = tile_m * SBM, n0 = tile_n * SBN;
+
+  DmaLoader<A_KMAJOR, SBM> la;
+  DmaLoader<B_KMAJOR, SBN> lb;
+  la.init(g.lda, m0, g.M, wave, lane);
+  lb.init(g.ldb, n0, g.N, wave, lane);
+  FragReaderF<A_KMAJOR, SBM> fra;
+  FragReaderF<B_KMAJOR, SBN> frb;
+  fra.init(wm * 32, lane);
+  frb.init(wn * 32, lane);
+
+  const float *Az = g.A + (long)z * g.sA;
+  const float *Bz = g.B + (long)z * g.sB;
+
+  float16v acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+  // K tiles [kt_base, kt_base + kt_end) belong to this workgroup
+  const int kt_base = SPLIT ? (int)((long)split * g.total_ktiles / g.splits) : 0;
+  const int kt_end = SPLIT ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
+  auto issue_tile = [&](int kt, int q) {
+    // instruction q of the 4 that move K tile kt (2 for A, then 2 for B)
+    const bool live = kt < kt_end;
+    const int ktc = live ? kt + kt_base : 0;
+    const int r = ktc / g.ktiles_per_r;
+    const int kt_in_r = ktc - r * g.ktiles_per_r;
+    const uint32_t stage = lds_base + (uint32_t)(kt & 1) * kStage64;
+    if (q < 2) la.issue(make_rsrc_words(Az + (long)r * g.rA, d.a_bytes), stage, wave, q, kt_in_r, g.K, live);
+    else lb.issue(make_rsrc_words(Bz + (long)r * g.rB, d.b_bytes), stage + kRegion64, wave, q - 2, kt_in_r, g.K, live);
+  };
+
+#pragma unroll
+  for (int q = 0; q < 4; ++q) issue_tile(0, q);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) issue_tile(1, q);
+  asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // tile 0 has landed
+  __syncthreads();
+
+  // fragments of one group of 8 k (block 0 of the readers' two), double-buffered as above
+  float fa[2][2][4], fb[2][2][4];
+  constexpr int kReadsA = A_KMAJOR ? 1 : 4, kReadsB = B_KMAJOR ? 1 : 4;
+#pragma unroll
+  for (int q = 0; q < kReadsA; ++q) fra.read_one(lds, 0, q, fa[0]);
+#pragma unroll
+  for (int q = 0; q < kReadsB; ++q) frb.read_one(lds + kRegion64, 0, q, fb[0]);
+
+  for (int kt = 0; kt < kt_end; ++kt) {
+    const int stage = kt & 1;
+#pragma unroll
+    for (int gk = 0; gk < 4; ++gk) {
+      const int cur = gk & 1, nxt = cur ^ 1;
+      const unsigned char *src = lds + (gk < 3 ? stage : stage ^ 1) * kStage64;
+      const int ngk = gk < 3 ? gk + 1 : 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // rows of the instruction's result follow n, its columns follow m
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][0][e], fa[cur][0][e], acc, 0, 0, 0);
+        if (e < kReadsA) fra.read_one(src, ngk, e, fa[nxt]);
+        if (e < kReadsB) frb.read_one(src + kRegion64, ngk, e, fb[nxt]);
+        // K tile kt+2 refills this stage once everybody has left it
+        if (gk == 3) issue_tile(kt + 2, e);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (gk == 2) {
+        // own loads of tile kt+1 have landed and own reads of this stage are
+        // done; behind the barrier that holds for every wave
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  float *Cz = g.C + (long)z * g.sC;
+  const bool interior = m0 + SBM <= g.M && n0 + SBN <= g.N;
+  const int row0 = m0 + wm * 32, col0 = n0 + wn * 32;
+  int ns[16];
+  float vals[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    ns[v] = 8 * (v / 4) + (v % 4);
+    vals[v] = acc[v];
+  }
+  if constexpr (SPLIT) {
+    if (g.atomic == 2) {
+      __shared__ uint32_t last_flag;
+      store_partial<16>(g, z, split, row0, col0, lane, ns, vals);
+      if (!last_of_tile(g, (z * g.tiles_n + tile_n) * g.tiles_m + tile_m, &last_flag)) return;
+      sum_partials<16>(g, z, row0, col0, lane, ns, vals);
+      emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, 0, g.accumulate);
+      return;
+    }
+  }
+  emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, SPLIT ? g.atomic : 0, g.accumulate);
+}
+
+// Fills the argument block shared by both tile sizes.
+static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, long a_bytes, long b_bytes,
+                      phip_ctx *ctx, LdsArgs *d) {
+  GemmArgs &a = d->g;
+  a.A = static_cast<const float *>(p.A);
+  a.B = static_cast<const float *>(p.B);
+  a.C = static_cast<float *>(p.C);
+  a.M = p.M; a.N = p.N; a.K = p.K;
+  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
+  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
+  a.rA = p.rA; a.rB = p.rB;
+  a.tiles_m = (p.M + side - 1) / side;
+  a.tiles_n = (p.N + side - 1) / side;
+  a.splits = (int)splits;
+  a.ktiles_per_r = (p.K + LBK - 1) / LBK;
+  a.total_ktiles = (int)total_ktiles;
+  a.atomic = splits > 1;
+  a.accumulate = p.accumulate ? 1 : 0;
+  a.partial = nullptr;
+  a.tickets = ctx->tile_tickets;
+  d->a_bytes = (uint32_t)a_bytes;
+  d->b_bytes = (uint32_t)b_bytes;
+}
+
+// A split overwriting product: fp32 partial tiles in scratch memory, summed by the last workgroup of
+// each tile; without room for them, a zero fill and atomics.  *block is the scratch memory, if any.
+static int prepare_split_overwrite(phip_ctx *ctx, const Gemm &p, long tiles, long splits, LdsArgs *d, void **block) {
+  GemmArgs &a = d->g;
+  const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
+  if (tiles <= kTicketSlots && bytes <= (size_t)(256L << 20) && phip_pool_alloc(ctx, bytes, block, nullptr) == PHIP_OK) {
+    a.atomic = 2;
+    a.partial = static_cast<float *>(*block);
+    return PHIP_OK;
+  }
+  *block = nullptr;
+  const int cus = ctx->prop.multiProcessorCount;
+  const long total = (long)p.M * p.N * p.batch;
+  long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+  if (blocks > cus * 8L) blocks = cus * 8L;
+  hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N, p.ldc,
+                     p.sC, p.batch);
+  PHIP_LAUNCH_CHECK();
+  return PHIP_OK;
+}
+
 }  // namespace
 
 // Large, 16-byte-aligned problems: at least one 128 x 128 tile per CU, or an
-// eighth of that with a K long enough to be cut between workgroups.  Sets
-// *handled when it launched.
+// eighth of that with a K long enough to be cut between workgroups; else
+// 64 x 64 tiles when those fill the chip.  Sets *handled when it launched.
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
   auto aligned = [](const void *ptr, long ld, long s, long r) {
@@ -181,20 +352,23 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   if ((p.a_kmajor ? p.K : p.M) != p.lda || (p.b_kmajor ? p.K : p.N) != p.ldb) return PHIP_OK;
   const long a_bytes = 4L * p.M * p.K, b_bytes = 4L * p.N * p.K;
   if (a_bytes >= (1L << 31) || b_bytes >= (1L << 31)) return PHIP_OK;
-  const long tiles = (long)((p.M + LBM - 1) / LBM) * ((p.N + LBN - 1) / LBN) * p.batch;
-  const int cus = ctx->prop.multiProcessorCount;
-  if ((long)p.K * p.rbatch <= 128 || tiles > 0x7fffffffL) return PHIP_OK;
+  if ((long)p.K * p.rbatch <= 128) return PHIP_OK;
   if (p.a_kmajor && !p.b_kmajor) return PHIP_OK;
+  const int cus = ctx->prop.multiProcessorCount;
   const long total_ktiles = (long)((p.K + LBK - 1) / LBK) * p.rbatch;
-  // Fewer tiles than CUs: worth it for a long K (from 2048) cut into ranges of at least 8 K tiles, when the
-  // tiles alone fill between an eighth and three quarters of the CUs (measured on M, N in 512 .. 4096: with
-  // a shorter K, or more tiles, the staged 64 x 64 tiles are as fast or faster).  The number of ranges
-  // minimises a small cost model fitted to those measurements: a fixed cost per workgroup, the time of a K
-  // tile when a workgroup has its CU to itself or shares it with a second one, and the exchange of the
-  // partial results, which grows with the number of ranges.
+  auto tiles_of = [&](int side) { return (long)((p.M + side - 1) / side) * ((p.N + side - 1) / side) * p.batch; };
+
+  // ---- 128 x 128 tiles
+  int side = LBM;
+  long tiles = tiles_of(LBM);
   long splits = 1;
-  if (tiles < cus) {
-    if (total_ktiles < 64 || tiles * 8 < cus || tiles * 4 >= cus * 3L) return PHIP_OK;
+  bool take = tiles >= cus && tiles <= 0x7fffffffL;
+  if (!take && tiles < cus && total_ktiles >= 64 && tiles * 8 >= cus && tiles * 4 < cus * 3L) {
+    // Fewer tiles than CUs: worth it for a long K (from 2048) cut into ranges of at least 8 K tiles, when the
+    // tiles alone fill between an eighth and three quarters of the CUs (measured on M, N in 512 .. 4096).  The
+    // number of ranges minimises a small cost model fitted to those measurements: a fixed cost per workgroup,
+    // the time of a K tile when a workgroup has its CU to itself or shares it with a second one, and the
+    // exchange of the partial results, which grows with the number of ranges.
     double best = 0.0;
     for (long s = 2; s <= 16 && s * 8 <= total_ktiles && tiles * s <= 2L * cus; ++s) {
       const double per_ktile = tiles * s <= cus ? 2.6 : 4.2;  // microseconds
@@ -204,66 +378,70 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
         splits = s;
       }
     }
-    if (splits < 2) return PHIP_OK;
+    take = splits >= 2;
+  }
+  // ---- 64 x 64 tiles
+  if (!take) {
+    // Measured on M, N in 256 .. 3072, K in 256 .. 1536 against the staged 64 x 64 tiles and the direct
+    // kernel: an overwriting product gains (15 - 35 %) when it is not split and has at least 3/4 tile per
+    // CU (the exchange of partial tiles costs more than the idle CUs); an accumulating product gains
+    // (10 - 25 %) from half a tile per CU on, its K cut into ranges of at least 8 tiles until the four
+    // places of every CU are filled, the tiles added with atomics.
+    side = SBM;
+    tiles = tiles_of(SBM);
+    const long least = p.accumulate ? cus / 2 : cus * 3L / 4;
+    if (tiles < least || tiles > 0x7fffffffL || 2L * p.M * p.N * p.batch < tiles * SBM * SBN) return PHIP_OK;
+    splits = 1;
+    if (p.accumulate && tiles < 4L * cus) {
+      splits = 4L * cus / tiles;
+      if (splits > total_ktiles / 8) splits = total_ktiles / 8;
+      if (splits > 16) splits = 16;
+      if (splits < 1) splits = 1;
+    }
+    take = true;
   }
 
   LdsArgs d;
-  GemmArgs &a = d.g;
-  a.A = static_cast<const float *>(p.A);
-  a.B = static_cast<const float *>(p.B);
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
-  a.tiles_m = (p.M + LBM - 1) / LBM;
-  a.tiles_n = (p.N + LBN - 1) / LBN;
-  a.splits = (int)splits;
-  a.ktiles_per_r = (p.K + LBK - 1) / LBK;
-  a.total_ktiles = (int)total_ktiles;
-  a.atomic = splits > 1;
-  a.accumulate = p.accumulate ? 1 : 0;
-  a.partial = nullptr;
-  a.tickets = ctx->tile_tickets;
-  d.a_bytes = (uint32_t)a_bytes;
-  d.b_bytes = (uint32_t)b_bytes;
-
-  // A split overwriting product: fp32 partial tiles in scratch memory, summed by the last workgroup of
-  // each tile; without room for them, a zero fill and atomics.
+  fill_args(p, side, splits, total_ktiles, a_bytes, b_bytes, ctx, &d);
   void *block = nullptr;
   if (splits > 1 && !p.accumulate) {
-    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
-    if (tiles <= kTicketSlots && bytes <= (size_t)(256L << 20) && phip_pool_alloc(ctx, bytes, &block, nullptr) == PHIP_OK) {
-      a.atomic = 2;
-      a.partial = static_cast<float *>(block);
-    } else {
-      const long total = (long)p.M * p.N * p.batch;
-      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-      if (blocks > cus * 8L) blocks = cus * 8L;
-      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N,
-                         p.ldc, p.sC, p.batch);
-      PHIP_LAUNCH_CHECK();
-    }
+    const int rc0 = prepare_split_overwrite(ctx, p, tiles, splits, &d, &block);
+    if (rc0 != PHIP_OK) return rc0;
   }
 
   int rc = PHIP_OK;
+  const unsigned grid = (unsigned)(tiles * splits);
 #define PHIP_LDS(SLOT, AK, BKM, SP)                                                                          \
   do {                                                                                                       \
     auto kern = gemm_f32_lds_kernel<AK, BKM, SP>;                                                            \
     rc = raise_lds_limit(ctx, SLOT + (SP ? 3 : 0), reinterpret_cast<const void *>(kern), kLdsBytes);         \
-    if (rc == PHIP_OK)                                                                                       \
-      hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * splits)), dim3(kThreads), kLdsBytes, ctx->stream, d); \
+    if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, ctx->stream, d);      \
   } while (0)
-  if (splits > 1) {
-    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, true);
-    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, true);
-    else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, true);
+#define PHIP_LDS64(AK, BKM, SP)                                                                              \
+  hipLaunchKernelGGL((gemm_f32_lds64_kernel<AK, BKM, SP>), dim3(grid), dim3(kThreads), kLds64Bytes, ctx->stream, d)
+  if (side == LBM) {
+    if (splits > 1) {
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, true);
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, true);
+      else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, true);
+    } else {
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, false);
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, false);
+      else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, false);
+    }
   } else {
-    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, false);
-    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, false);
-    else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, false);
+    if (splits > 1) {
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64(false, true, true);
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64(false, false, true);
+      else PHIP_LDS64(true, true, true);
+    } else {
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64(false, true, false);
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64(false, false, false);
+      else PHIP_LDS64(true, true, false);
+    }
   }
 #undef PHIP_LDS
+#undef PHIP_LDS64
   if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();

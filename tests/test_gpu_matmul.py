@@ -300,7 +300,7 @@ def test_gradients_into_one_buffer(dev):
     assert norm_rel_err(tg.to_vector(), rga + rgb) <= F32_TOL
 
 
-# mid-size products with a long K (from 2048) and fewer 128 x 128 tiles than CUs: the large-tile
+# mid-size products: with a long K (from 2048) and fewer 128 x 128 tiles than CUs the large-tile
 # kernel with its K range cut between workgroups - forward (partial tiles and tickets), both
 # gradients (atomics), ragged edges, per-sample products, a contraction over the minibatch
 MIDSIZE_F32 = [  # di, dj, dk, ba, bb
@@ -310,6 +310,10 @@ MIDSIZE_F32 = [  # di, dj, dk, ba, bb
     (1028, 1100, 2052, 1, 1),
     (520, 2080, 300, 3, 3),
     (700, 1040, 520, 3, 1),
+    # shorter K: 64 x 64 tiles moved global -> LDS directly (forward unsplit, gradients split with atomics)
+    (1028, 520, 1100, 1, 1),
+    (400, 264, 400, 4, 4),
+    (400, 264, 400, 4, 1),
 ]
 
 
