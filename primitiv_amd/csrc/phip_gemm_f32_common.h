@@ -34,6 +34,22 @@ struct GemmArgs {
   uint32_t *tickets; // atomic == 2: one zeroed counter per output tile, left zeroed
 };
 
+// The fields of the argument block that restate the problem; tile counts, K
+// ranges and the split's exchange are the caller's.
+inline GemmArgs problem_args(const Gemm &p) {
+  GemmArgs a = {};
+  a.A = static_cast<const float *>(p.A);
+  a.B = static_cast<const float *>(p.B);
+  a.C = static_cast<float *>(p.C);
+  a.M = p.M; a.N = p.N; a.K = p.K;
+  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
+  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
+  a.rA = p.rA; a.rB = p.rB;
+  a.splits = 1;
+  a.accumulate = p.accumulate ? 1 : 0;
+  return a;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
 // Renumber them so that one XCD receives a contiguous run of tiles.
 __device__ inline int xcd_remap(int bid, int total) {

@@ -227,13 +227,7 @@ inline bool plan_direct(const phip_ctx *ctx, const Gemm &p, DirectPlan *plan) {
 
   DirectArgs &d = plan->d;
   GemmArgs &a = d.g;
-  a.A = static_cast<const float *>(p.A);
-  a.B = static_cast<const float *>(p.B);
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
+  a = problem_args(p);
   a.accumulate = p.accumulate ? 1 : 0;
   a.ktiles_per_r = 0;
   a.total_ktiles = 0;

@@ -296,13 +296,7 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
 static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, long a_bytes, long b_bytes,
                       phip_ctx *ctx, LdsArgs *d) {
   GemmArgs &a = d->g;
-  a.A = static_cast<const float *>(p.A);
-  a.B = static_cast<const float *>(p.B);
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
+  a = problem_args(p);
   a.tiles_m = (p.M + side - 1) / side;
   a.tiles_n = (p.N + side - 1) / side;
   a.splits = (int)splits;

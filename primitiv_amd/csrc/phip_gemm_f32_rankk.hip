@@ -202,13 +202,7 @@ int gemm_f32_rankk(phip_ctx *ctx, const Gemm &p, bool *handled) {
 
   LdsArgs d;
   GemmArgs &a = d.g;
-  a.A = static_cast<const float *>(p.A);
-  a.B = static_cast<const float *>(p.B);
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
+  a = problem_args(p);
   a.tiles_m = (p.M + RBM - 1) / RBM;
   a.tiles_n = (p.N + RBN - 1) / RBN;
   a.splits = 1;

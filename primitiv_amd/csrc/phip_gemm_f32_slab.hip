@@ -313,13 +313,9 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
 
   LdsArgs d;
   GemmArgs &a = d.g;
-  a.A = static_cast<const float *>(p.A);
+  a = problem_args(p);
   a.B = b_ptr;
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = b_ld; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
+  a.ldb = b_ld;
   a.tiles_m = (p.M + TBM - 1) / TBM;
   a.tiles_n = 1;
   a.splits = (int)splits;

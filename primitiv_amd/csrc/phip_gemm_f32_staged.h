@@ -301,13 +301,7 @@ struct StagedPlan {
 
 inline void plan_staged(const phip_ctx *ctx, const Gemm &p, StagedPlan *plan) {
   GemmArgs &a = plan->a;
-  a.A = static_cast<const float *>(p.A);
-  a.B = static_cast<const float *>(p.B);
-  a.C = static_cast<float *>(p.C);
-  a.M = p.M; a.N = p.N; a.K = p.K;
-  a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
-  a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
-  a.rA = p.rA; a.rB = p.rB;
+  a = problem_args(p);
   a.accumulate = p.accumulate ? 1 : 0;
   a.partial = nullptr;
   a.tickets = nullptr;
