@@ -17,13 +17,8 @@ int launch_tile(phip_ctx *ctx, const Gemm &p, const StagedPlan &plan) {
   if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
 
   if (a.atomic && !p.accumulate) {
-    const int cus = ctx->prop.multiProcessorCount;
-    const long total = (long)p.M * p.N * p.batch;
-    long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-    if (blocks > cus * 8L) blocks = cus * 8L;
-    hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream,
-                       a.C, p.M, p.N, p.ldc, p.sC, p.batch);
-    PHIP_LAUNCH_CHECK();
+    const int rc = zero_c(ctx, p);
+    if (rc != PHIP_OK) return rc;
   }
 
   const bool vec_a = plan.vec_a, vec_b = plan.vec_b;

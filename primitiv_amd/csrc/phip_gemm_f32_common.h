@@ -204,6 +204,48 @@ __attribute__((unused)) __global__ __launch_bounds__(kThreads) void zero_c_kerne
   }
 }
 
+// Pool memory that goes back when the launches that use it have been enqueued
+// (the stream is in order, so the block may be handed out again behind them).
+struct Scratch {
+  phip_ctx *ctx;
+  void *ptr = nullptr;
+  explicit Scratch(phip_ctx *c) : ctx(c) {}
+  ~Scratch() {
+    if (ptr) phip_pool_free(ctx, ptr);
+  }
+  Scratch(const Scratch &) = delete;
+  Scratch &operator=(const Scratch &) = delete;
+};
+
+inline int zero_c(phip_ctx *ctx, const Gemm &p) {
+  const int cus = ctx->prop.multiProcessorCount;
+  const long total = (long)p.M * p.N * p.batch;
+  long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
+  if (blocks > cus * 8L) blocks = cus * 8L;
+  hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, static_cast<float *>(p.C),
+                     p.M, p.N, p.ldc, p.sC, p.batch);
+  PHIP_LAUNCH_CHECK();
+  return PHIP_OK;
+}
+
+// An overwriting product whose K is split between `a->splits` workgroups per
+// tile (a->atomic == 1 on entry): fp32 partial tiles in scratch memory, summed by
+// the last workgroup of each tile (a->atomic = 2: no zero fill of C, no atomics
+// on it, one launch, the same bits on every run); without room for them, or
+// with more tiles than tickets, a zero fill of C and atomics.
+inline int prepare_split_overwrite(phip_ctx *ctx, const Gemm &p, long tiles, size_t max_bytes, GemmArgs *a,
+                                   Scratch *partials) {
+  const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * a->splits;
+  if (tiles <= kTicketSlots && bytes <= max_bytes && phip_pool_alloc(ctx, bytes, &partials->ptr, nullptr) == PHIP_OK) {
+    a->atomic = 2;
+    a->partial = static_cast<float *>(partials->ptr);
+    a->tickets = ctx->tile_tickets;
+    return PHIP_OK;
+  }
+  partials->ptr = nullptr;
+  return zero_c(ctx, p);
+}
+
 }  // namespace
 }  // namespace phip
 

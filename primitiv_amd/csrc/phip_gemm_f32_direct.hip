@@ -18,25 +18,11 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, const DirectPlan &plan) {
   GemmArgs &a = d.g;
   const long grid = plan.grid;
   if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
-  // An overwriting product that is split leaves fp32 partial tiles in scratch memory and lets the last
-  // workgroup of each tile add them (no zero fill of C, no atomics on it, one launch); the atomics
-  // remain for an accumulating product and as the fallback.
-  void *block = nullptr;
+  Scratch partials(ctx);
   if (a.atomic && !p.accumulate) {
-    const long tiles = (long)a.tiles_m * a.tiles_n * p.batch;
-    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * a.splits;
-    if (tiles <= kTicketSlots && bytes <= (size_t)(64L << 20) && phip_pool_alloc(ctx, bytes, &block, nullptr) == PHIP_OK) {
-      a.atomic = 2;
-      a.partial = static_cast<float *>(block);
-    } else {
-      const int cus = ctx->prop.multiProcessorCount;
-      const long total = (long)p.M * p.N * p.batch;
-      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-      if (blocks > cus * 8L) blocks = cus * 8L;
-      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N,
-                         p.ldc, p.sC, p.batch);
-      PHIP_LAUNCH_CHECK();
-    }
+    const int rc = prepare_split_overwrite(ctx, p, (long)a.tiles_m * a.tiles_n * p.batch, (size_t)(64L << 20), &a,
+                                           &partials);
+    if (rc != PHIP_OK) return rc;
   }
   const bool vec_a = plan.vec_a, vec_b = plan.vec_b;
 #define PHIP_DIRECT_V(AK, BKM, VVA, VVB)                                                                 \
@@ -53,11 +39,9 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, const DirectPlan &plan) {
     else if (vec_b) PHIP_DIRECT_V(true, true, 1, 4);
     else PHIP_DIRECT_V(true, true, 1, 1);
   } else {
-    if (block) phip_pool_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
 #undef PHIP_DIRECT_V
-  if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
 }

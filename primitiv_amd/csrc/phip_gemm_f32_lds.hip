@@ -310,27 +310,6 @@ static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, l
   d->b_bytes = (uint32_t)b_bytes;
 }
 
-// A split overwriting product: fp32 partial tiles in scratch memory, summed by the last workgroup of
-// each tile; without room for them, a zero fill and atomics.  *block is the scratch memory, if any.
-static int prepare_split_overwrite(phip_ctx *ctx, const Gemm &p, long tiles, long splits, LdsArgs *d, void **block) {
-  GemmArgs &a = d->g;
-  const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
-  if (tiles <= kTicketSlots && bytes <= (size_t)(256L << 20) && phip_pool_alloc(ctx, bytes, block, nullptr) == PHIP_OK) {
-    a.atomic = 2;
-    a.partial = static_cast<float *>(*block);
-    return PHIP_OK;
-  }
-  *block = nullptr;
-  const int cus = ctx->prop.multiProcessorCount;
-  const long total = (long)p.M * p.N * p.batch;
-  long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-  if (blocks > cus * 8L) blocks = cus * 8L;
-  hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N, p.ldc,
-                     p.sC, p.batch);
-  PHIP_LAUNCH_CHECK();
-  return PHIP_OK;
-}
-
 }  // namespace
 
 // Large, 16-byte-aligned problems: at least one 128 x 128 tile per CU, or an
@@ -397,9 +376,9 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
 
   LdsArgs d;
   fill_args(p, side, splits, total_ktiles, a_bytes, b_bytes, ctx, &d);
-  void *block = nullptr;
+  Scratch partials(ctx);
   if (splits > 1 && !p.accumulate) {
-    const int rc0 = prepare_split_overwrite(ctx, p, tiles, splits, &d, &block);
+    const int rc0 = prepare_split_overwrite(ctx, p, tiles, (size_t)(256L << 20), &d.g, &partials);
     if (rc0 != PHIP_OK) return rc0;
   }
 
@@ -436,7 +415,6 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   }
 #undef PHIP_LDS
 #undef PHIP_LDS64
-  if (block) phip_pool_free(ctx, block);  // the stream is in order: reusable behind this launch
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
   *handled = true;

@@ -238,19 +238,6 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_slab_kernel(const LdsArg
   }
 }
 
-// Pool memory that goes back when the launches that use it have been enqueued (the stream is in order, so
-// the block may be handed out again behind them).
-struct Scratch {
-  phip_ctx *ctx;
-  void *ptr = nullptr;
-  explicit Scratch(phip_ctx *c) : ctx(c) {}
-  ~Scratch() {
-    if (ptr) phip_pool_free(ctx, ptr);
-  }
-  Scratch(const Scratch &) = delete;
-  Scratch &operator=(const Scratch &) = delete;
-};
-
 // dst (rows of `kp` floats, 16-byte aligned) = the `n` rows of `k` floats of src (leading dimension ld),
 // each followed by zeros
 __global__ __launch_bounds__(kThreads) void pad_rows_kernel(const float *src, long ld, float *dst, int kp, int n, int k) {
@@ -328,24 +315,10 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_size;
 
-  // An overwriting product that is split leaves fp32 partial tiles in scratch memory and lets the last
-  // workgroup of each tile add them; the atomics remain for an accumulating product and as the fallback
-  // (then behind a zero fill of C).
   Scratch partials(ctx);
   if (a.atomic && !p.accumulate) {
-    const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * splits;
-    if (tiles <= kTicketSlots && bytes <= (size_t)(64L << 20) && phip_pool_alloc(ctx, bytes, &partials.ptr, nullptr) == PHIP_OK) {
-      a.atomic = 2;
-      a.partial = static_cast<float *>(partials.ptr);
-      a.tickets = ctx->tile_tickets;
-    } else {
-      const long total = (long)p.M * p.N * p.batch;
-      long blocks = (total + kThreads * 4 - 1) / (kThreads * 4);
-      if (blocks > cus * 8L) blocks = cus * 8L;
-      hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, a.C, p.M, p.N, p.ldc,
-                         p.sC, p.batch);
-      PHIP_LAUNCH_CHECK();
-    }
+    const int rc = prepare_split_overwrite(ctx, p, tiles, (size_t)(64L << 20), &a, &partials);
+    if (rc != PHIP_OK) return rc;
   }
   const long grid = tiles * splits;
 #define PHIP_SLAB_G(SLOT, AK, BKM, VB)                                                              \
