@@ -236,11 +236,8 @@ inline bool plan_direct(const phip_ctx *ctx, const Gemm &p, DirectPlan *plan) {
   d.chunks_per_r = (p.K + 7) / 8;
   d.total_chunks = d.chunks_per_r * p.rbatch;
 
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
-  };
-  plan->vec_a = p.a_kmajor && aligned(p.A, p.lda, p.sA, p.rA) && p.K % 4 == 0;
-  plan->vec_b = p.b_kmajor && aligned(p.B, p.ldb, p.sB, p.rB) && p.K % 4 == 0;
+  plan->vec_a = p.a_kmajor && rows_aligned16(p.A, 4, p.lda, p.sA, p.rA) && p.K % 4 == 0;
+  plan->vec_b = p.b_kmajor && rows_aligned16(p.B, 4, p.ldb, p.sB, p.rB) && p.K % 4 == 0;
 
   // A k-contiguous operand that cannot be read 16 bytes at a time would be
   // fetched as 4-byte loads scattered over 32 rows; the staged kernel reads

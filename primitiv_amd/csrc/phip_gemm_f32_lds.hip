@@ -317,10 +317,7 @@ static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, l
 // 64 x 64 tiles when those fill the chip.  Sets *handled when it launched.
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
-  };
-  if (!aligned(p.A, p.lda, p.sA, p.rA) || !aligned(p.B, p.ldb, p.sB, p.rB)) return PHIP_OK;
+  if (!rows_aligned16(p.A, 4, p.lda, p.sA, p.rA) || !rows_aligned16(p.B, 4, p.ldb, p.sB, p.rB)) return PHIP_OK;
   // the contiguous extent of a dense operand is its leading dimension
   if ((p.a_kmajor ? p.K : p.M) != p.lda || (p.b_kmajor ? p.K : p.N) != p.ldb) return PHIP_OK;
   const long a_bytes = 4L * p.M * p.K, b_bytes = 4L * p.N * p.K;

@@ -184,11 +184,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_rankk_kernel(const LdsAr
 int gemm_f32_rankk(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
   if (p.a_kmajor || p.b_kmajor || p.rbatch != 1 || p.K > kKTiles * LBK) return PHIP_OK;
-  auto aligned = [](const void *ptr, long ld, long s) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0;
-  };
-  if (!aligned(p.A, p.lda, p.sA) || !aligned(p.C, p.ldc, p.sC)) return PHIP_OK;
-  const bool vec_b = aligned(p.B, p.ldb, p.sB);
+  if (!rows_aligned16(p.A, 4, p.lda, p.sA) || !rows_aligned16(p.C, 4, p.ldc, p.sC)) return PHIP_OK;
+  const bool vec_b = rows_aligned16(p.B, 4, p.ldb, p.sB);
   // rows of B that are 8-byte aligned can still move two columns per lane
   if (!vec_b && (reinterpret_cast<uintptr_t>(p.B) % 8 != 0 || p.ldb % 2 != 0 || p.sB % 2 != 0)) return PHIP_OK;
   // the contiguous extent of a dense operand is its leading dimension

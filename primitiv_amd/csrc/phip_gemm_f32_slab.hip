@@ -253,13 +253,10 @@ __global__ __launch_bounds__(kThreads) void pad_rows_kernel(const float *src, lo
 // Narrow outputs over a large streamed operand.  Sets *handled when it launched.
 int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
-  };
   if (p.N > TBN) return PHIP_OK;
-  if (!aligned(p.A, p.lda, p.sA, p.rA)) return PHIP_OK;
+  if (!rows_aligned16(p.A, 4, p.lda, p.sA, p.rA)) return PHIP_OK;
   // a k-contiguous B may have rows that are only 4-byte aligned: it is then moved by 4-byte loads
-  const bool vec_b = aligned(p.B, p.ldb, p.sB, p.rB);
+  const bool vec_b = rows_aligned16(p.B, 4, p.ldb, p.sB, p.rB);
   if (!vec_b && !p.b_kmajor) return PHIP_OK;
   // the contiguous extent of a dense operand is its leading dimension
   if ((p.a_kmajor ? p.K : p.M) != p.lda || (p.b_kmajor ? p.K : p.N) != p.ldb) return PHIP_OK;

@@ -306,13 +306,10 @@ inline void plan_staged(const phip_ctx *ctx, const Gemm &p, StagedPlan *plan) {
   a.partial = nullptr;
   a.tickets = nullptr;
 
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 4 == 0 && s % 4 == 0 && r % 4 == 0;
-  };
   // 16-byte loads need aligned rows and a contiguous-axis extent that is a
   // multiple of 4 (so that no vector straddles the matrix edge).
-  plan->vec_a = aligned(p.A, p.lda, p.sA, p.rA) && (p.a_kmajor ? p.K : p.M) % 4 == 0;
-  plan->vec_b = aligned(p.B, p.ldb, p.sB, p.rB) && (p.b_kmajor ? p.K : p.N) % 4 == 0;
+  plan->vec_a = rows_aligned16(p.A, 4, p.lda, p.sA, p.rA) && (p.a_kmajor ? p.K : p.M) % 4 == 0;
+  plan->vec_b = rows_aligned16(p.B, 4, p.ldb, p.sB, p.rB) && (p.b_kmajor ? p.K : p.N) % 4 == 0;
 
   const int cus = ctx->prop.multiProcessorCount;
   auto tiles = [&](int bm, int bn) {

@@ -461,11 +461,8 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
   a.accumulate = p.accumulate ? 1 : 0;
   a.vec_c = reinterpret_cast<uintptr_t>(p.C) % 16 == 0 && p.M % 8 == 0 && p.ldc % 8 == 0 && p.sC % 8 == 0;
 
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 8 == 0 && s % 8 == 0 && r % 8 == 0;
-  };
   // 16-byte loads per operand: aligned rows (the loaders check the ragged edge per vector)
-  const bool vec_a = aligned(p.A, p.lda, p.sA, p.rA), vec_b = aligned(p.B, p.ldb, p.sB, p.rB);
+  const bool vec_a = rows_aligned16(p.A, 8, p.lda, p.sA, p.rA), vec_b = rows_aligned16(p.B, 8, p.ldb, p.sB, p.rB);
 
   const int cus = ctx->prop.multiProcessorCount;
   auto tiles = [&](int bm, int bn) {

@@ -537,13 +537,10 @@ int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
 // kernel (aligned, big enough, each operand sample under 2 GiB).
 int gemm_h16_big(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   *handled = false;
-  auto aligned = [](const void *ptr, long ld, long s, long r) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && ld % 8 == 0 && s % 8 == 0 && r % 8 == 0;
-  };
-  if (!aligned(p.A, p.lda, p.sA, p.rA) || !aligned(p.B, p.ldb, p.sB, p.rB)) return PHIP_OK;
+  if (!rows_aligned16(p.A, 8, p.lda, p.sA, p.rA) || !rows_aligned16(p.B, 8, p.ldb, p.sB, p.rB)) return PHIP_OK;
   if ((p.a_kmajor ? p.K : p.M) % 8 != 0 || (p.b_kmajor ? p.K : p.N) % 8 != 0) return PHIP_OK;
   // C is written 8 rows (16 bytes) at a time
-  if (!aligned(p.C, p.ldc, p.sC, 0) || p.M % 8 != 0) return PHIP_OK;
+  if (!rows_aligned16(p.C, 8, p.ldc, p.sC, 0) || p.M % 8 != 0) return PHIP_OK;
   // the contiguous extent of a dense operand is its leading dimension
   if ((p.a_kmajor ? p.K : p.M) != p.lda || (p.b_kmajor ? p.K : p.N) != p.ldb) return PHIP_OK;
   const long a_bytes = 2L * p.M * p.K, b_bytes = 2L * p.N * p.K;

@@ -122,6 +122,13 @@ struct Gemm {
 
 enum class Elem { F32, F16, BF16 };
 
+// True when an operand can be moved 16 bytes at a time: its base is 16-byte
+// aligned and its leading dimension and strides are multiples of `per16`
+// elements (4 for fp32, 8 for 16-bit storage).
+inline bool rows_aligned16(const void *ptr, int per16, long ld, long s = 0, long r = 0) {
+  return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && ld % per16 == 0 && s % per16 == 0 && r % per16 == 0;
+}
+
 int gemm_f32(phip_ctx *ctx, const Gemm &g);
 int gemm_f32_direct(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &g, bool *handled);
