@@ -135,3 +135,40 @@ def test_shape_rules():
                 ([5, 5, 1, 2], 1, 1, 0, 0, 1, 1)):
         with pytest.raises(ValueError):
             oracle.shape_pool2d(*bad)
+
+
+def test_host_shape_rules_agree_with_the_oracle():
+    # the Python mirror's shape_ops.conv2d / pool2d (host logic, no GPU) against the oracle's restatement,
+    # valid and invalid arguments alike
+    import itertools
+    import primitiv_amd as pa
+    S = pa.Shape
+    xs = [([5, 5], 1), ([5, 4, 3], 2), ([7], 1), ([], 1), ([6, 6, 2], 3)]
+    ws = [([2, 2], 1), ([3, 2, 3, 4], 1), ([1], 2), ([], 1), ([2, 3, 2, 5], 3), ([9, 1], 1)]
+    args = [(0, 0, 1, 1, 1, 1), (1, 2, 2, 1, 1, 2), (0, 1, 1, 0, 1, 1), (2, 0, 3, 2, 0, 1), (3, 3, 1, 1, 3, 3)]
+    agree = 0
+    for (xd, bx), (wd, bw), a in itertools.product(xs, ws, args):
+        try:
+            want = oracle.shape_conv2d(xd, bx, wd, bw, *a)
+        except ValueError:
+            want = None
+        try:
+            got = pa.shape_ops.conv2d(S(xd, bx), S(wd, bw), *a)
+            got = ([got[0], got[1], got[2]], got.batch())
+        except pa.Error:
+            got = None
+        assert got == want, (xd, bx, wd, bw, a)
+        agree += want is not None
+    assert agree > 20
+    for (xd, bx), a in itertools.product(xs, [(2, 2, 0, 0, 2, 2), (3, 1, 1, 0, 1, 1), (0, 1, 0, 0, 1, 1), (2, 2, 1, 1, 0, 1),
+                                           (9, 9, 1, 1, 1, 1), (1, 1, 0, 0, 3, 2)]):
+        try:
+            want = oracle.shape_pool2d(xd, *a)
+        except ValueError:
+            want = None
+        try:
+            got = pa.shape_ops.pool2d(S(xd, bx), *a)
+            got = [got[0], got[1], got[2]]
+        except pa.Error:
+            got = None
+        assert got == want, (xd, a)
