@@ -16,12 +16,14 @@
 namespace phip {
 namespace {
 
-constexpr int kStaged = 64;  // FIRST: 4 or 8 = chunks in flight of the direct kernel, or this
+// FIRST: 4 or 8 = chunks in flight of the direct kernel, or the staged 64 x 64 tiles with B moved 16 or
+// (rows not 16-byte aligned: a hidden size such as 650) 4 bytes at a time
+constexpr int kStaged = 64, kStagedB1 = 65;
 
 template <int FIRST>
 constexpr int pair_lds_floats() {
   constexpr int direct = kDirectRedFloats<1, 1, 4>;
-  constexpr int staged = FIRST == kStaged ? staged_lds_floats<64, 64, 32, 2, 2, 1>() : 0;
+  constexpr int staged = FIRST >= kStaged ? staged_lds_floats<64, 64, 32, 2, 2, 1>() : 0;
   return direct > staged ? direct : staged;
 }
 
@@ -33,6 +35,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_pair_kernel(const Direct
   const int bid = blockIdx.x;
   if (bid < first_blocks) {
     if constexpr (FIRST == kStaged) staged_tile<64, 64, 32, 2, 2, 1, false, false, 4, 4>(first.g, lds, bid, first_blocks);
+    else if constexpr (FIRST == kStagedB1) staged_tile<64, 64, 32, 2, 2, 1, false, false, 4, 1>(first.g, lds, bid, first_blocks);
     else direct_tile<1, 1, FIRST, false, false, 1, 1, 4>(first, lds, &last_flag, bid, first_blocks);
   } else if (bid >= first_padded) {
     // the second problem starts at a multiple of 8 so that its workgroups meet the XCDs in the same order
@@ -69,12 +72,12 @@ int gemm_f32_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *ha
     if ((long)first.K * first.rbatch > 128 || tiles128 * 2 >= cus) return PHIP_OK;
     StagedPlan sp;
     plan_staged(ctx, first, &sp);
-    if (sp.shape != StagedShape::k64x64x32 || !sp.vec_a || !sp.vec_b) return PHIP_OK;
+    if (sp.shape != StagedShape::k64x64x32 || !sp.vec_a) return PHIP_OK;
     p1.d.g = sp.a;
     p1.d.chunks_per_r = 0;
     p1.d.total_chunks = 0;
     p1.grid = sp.grid;
-    kind = kStaged;
+    kind = sp.vec_b ? kStaged : kStagedB1;
   }
   const long padded = (p1.grid + 7) / 8 * 8;
   if (padded + p2.grid > 0x7fffffffL) return PHIP_OK;
@@ -84,10 +87,12 @@ int gemm_f32_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *ha
                      ctx->stream, p1.d, p2.d, (int)p1.grid, (int)padded)
   if (p2.u == 8) {
     if (kind == kStaged) PHIP_PAIR(kStaged, 8);
+    else if (kind == kStagedB1) PHIP_PAIR(kStagedB1, 8);
     else if (kind == 8) PHIP_PAIR(8, 8);
     else PHIP_PAIR(4, 8);
   } else {
     if (kind == kStaged) PHIP_PAIR(kStaged, 4);
+    else if (kind == kStagedB1) PHIP_PAIR(kStagedB1, 4);
     else if (kind == 8) PHIP_PAIR(8, 4);
     else PHIP_PAIR(4, 4);
   }

@@ -262,6 +262,7 @@ PAIRED_F32 = [  # di, dj, dk, ba, bb
     (64, 64, 8, 9, 1),
     (132, 260, 24, 6, 6),
     (1024, 1024, 1, 1, 8),
+    (2600, 650, 1, 1, 64),      # an LSTM's gates with 650 hidden units: rows of b^T are not 16-byte aligned
 ]
 
 
