@@ -183,6 +183,58 @@ def test_random_shapes_h16(dev16, devbf16, which, ba, bb):
                 assert norm_rel_err(got, ref) <= tol, name + " " + tag
 
 
+def _drawn_dim(rng):
+    kind = int(rng.integers(0, 6))
+    if kind == 0:
+        return int(rng.integers(1, 20))
+    if kind == 1:
+        return int(rng.integers(1, 200))
+    if kind == 2:
+        return int(rng.integers(1, 90)) * 8
+    if kind == 3:
+        return int(rng.integers(100, 1400))
+    if kind == 4:
+        return int(rng.choice([64, 128, 256, 512, 1024, 650, 2600, 2048, 4096]))
+    return int(rng.integers(1000, 5000))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_drawn_dimensions_all_devices(dev, dev16, devbf16, seed):
+    # Dimensions drawn from tiny / odd / multiple-of-8 / layer-sized / long
+    # classes, independently per axis, so that a seed crosses most kernel
+    # choices and their edge handling.  Reference: float64 numpy on the values
+    # each device actually stores (gate: F32_TOL, H16_TOL of max|ref|).
+    rng = np.random.default_rng(9000 + seed)
+    for it in range(25):
+        di, dj, dk = (_drawn_dim(rng) for _ in range(3))
+        ba, bb = [(1, 1), (1, 1), (1, int(rng.integers(2, 6))), (int(rng.integers(2, 6)), 1), (3, 3)][
+            int(rng.integers(0, 5))]
+        bs = max(ba, bb)
+        while di * dj * dk * bs > 2e9 or max(di * dj * ba, dj * dk * bb, di * dk * bs) > 2e7:
+            if di >= dj and di >= dk:
+                di = di // 2 + 1
+            elif dj >= dk:
+                dj = dj // 2 + 1
+            else:
+                dk = dk // 2 + 1
+        a = rng.standard_normal(di * dj * ba).astype(np.float32)
+        b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+        gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+        ga0 = rng.standard_normal(a.size).astype(np.float32)
+        gb0 = rng.standard_normal(b.size).astype(np.float32)
+        for d, tol in ((dev, F32_TOL), (dev16, H16_TOL), (devbf16, H16_TOL)):
+            stored = [d.new_tensor_by_vector(pa.Shape(dims, n), v).to_vector().astype(np.float64)
+                      for dims, n, v in (([di, dj], ba, a), ([dj, dk], bb, b), ([di, dk], bs, gy),
+                                         ([di, dj], ba, ga0), ([dj, dk], bb, gb0))]
+            y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+            ry = np_matmul_fw(stored[0], stored[1], di, dj, dk, ba, bb)
+            dga, dgb = np_matmul_bw(stored[0], stored[1], stored[2], di, dj, dk, ba, bb)
+            tag = "%s draw %d shape (%d,%d,%d) batch (%d,%d)" % (type(d).__name__, it, di, dj, dk, ba, bb)
+            assert norm_rel_err(y, ry) <= tol, "y " + tag
+            assert norm_rel_err(ga, stored[3] + dga) <= tol, "ga " + tag
+            assert norm_rel_err(gb, stored[4] + dgb) <= tol, "gb " + tag
+
+
 # shapes that reach the fp32 128x128x32 global-to-LDS kernel (>= one tile per CU)
 # with ragged edges in every dimension (multiples of 4, not of 128 / 32)
 BIG_F32 = [  # di, dj, dk, ba, bb

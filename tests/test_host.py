@@ -32,6 +32,22 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.SIGNATURES)
 
 
+@pytest.mark.parametrize("compiler,std,lang", [("gcc", "-std=c99", "c"), ("g++", "-std=c++11", "c++")])
+def test_header_is_plain_c_and_cxx(tmp_path, compiler, std, lang):
+    """The boundary is a C ABI: the header must compile on its own as strict C99
+    (what cgo / ctypes-style bindings parse) and as C++11 (what primitiv uses)."""
+    import shutil
+    import subprocess
+    if not shutil.which(compiler):
+        pytest.skip(compiler + " not installed")
+    src = tmp_path / "include_only.c"
+    src.write_text('#include "phip.h"\nint main(void) { return 0; }\n')
+    cmd = [compiler, std, "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", lang,
+           "-I" + os.path.join(ROOT, "include"), str(src)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+
 def test_status_and_message_without_gpu():
     l = _lib.lib()
     assert l.phip_sync(None) == _lib.PHIP_ERR_INVALID_ARGUMENT
