@@ -1,9 +1,17 @@
 // Large-tile GEMM for 16-bit storage (fp16 / bf16, fp32 accumulation):
 // 256 x 256 x 64 tiles, one workgroup (4 wavefronts, each a 128 x 128 block of
-// 4 x 4 v_mfma_f32_32x32x16 tiles, 256 accumulator registers per lane) per CU,
+// 8 x 8 v_mfma_f32_16x16x32 tiles, 256 accumulator registers per lane) per CU,
 // two 64 KiB LDS stages.  Problems with too few such tiles for the chip take
-// 128 x 128 x 64 tiles instead (wavefronts of 2 x 2 blocks, two 32 KiB stages,
+// 128 x 128 x 64 tiles instead (wavefronts of 4 x 4 blocks, two 32 KiB stages,
 // two workgroups per CU): the same code with half the extents.
+//
+// The 16 x 16 x 32 instruction, not the 32 x 32 x 16 one: these kernels run at
+// the power limit, where the clock follows what the instructions draw, and a
+// register-only loop of the smaller shape settles a fifth higher (1.97 against
+// 1.63 GHz with fp16 operands).  Its price is a pipe that is busy for only 16
+// cycles per instruction while a wavefront issues one instruction every 4, so
+// the K loop is laid out with at most three other instructions between two of
+// them.
 //
 // Nothing is staged through registers and nothing is transposed by ALU work:
 //  * both operands are moved global -> LDS by buffer loads that write LDS
@@ -16,21 +24,23 @@
 // LDS rows are not padded (a load instruction fills 1 KiB of consecutive LDS);
 // bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row
 // each lane fetches.
+#include <type_traits>
+
 #include "phip_internal.h"
 #include "phip_types.h"
 
 namespace phip {
 namespace {
 
-typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int BK = 64;
-// WB = 32 x 32 blocks per wavefront and direction: 4 -> 256 x 256 tiles (one workgroup per CU),
-// 2 -> 128 x 128 tiles (two workgroups per CU) for problems with too few large tiles
+// WB = 32 rows (two blocks of 16) per wavefront and direction: 4 -> 256 x 256 tiles (one workgroup per
+// CU), 2 -> 128 x 128 tiles (two workgroups per CU) for problems with too few large tiles
 template <int WB> constexpr int kTile = 64 * WB;                  // rows = columns of a workgroup's tile
 template <int WB> constexpr int kRegion = kTile<WB> * BK * 2;     // bytes of one operand tile
 template <int WB> constexpr int kStage = 2 * kRegion<WB>;
@@ -60,14 +70,24 @@ __device__ inline int xcd_remap(int bid, int total) {
   return xcd * q + (xcd < rem ? xcd : rem) + idx;
 }
 
+// D = A . B for a 16 x 16 block over 32 k: lane l supplies row l % 16 of A (and
+// column l % 16 of B), k = 8 (l / 16) .. + 7, and receives rows 4 (l / 16) .. + 3
+// of column l % 16.
+//
+// Written as inline assembly with the accumulator tied to an AGPR tuple: left to
+// the register allocator, most of the 64 accumulators of a wavefront were
+// copied to a spare tuple before every instruction (the form whose result
+// must not overlap its addend).  The compiler therefore does not know these
+// are matrix instructions; the kernel keeps its own distance between the last
+// of them and the first ordinary read of an accumulator.
 template <bool BF16>
-__device__ inline float16v mfma(uint4v a, uint4v b, float16v c) {
-  if constexpr (BF16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c, 0, 0, 0);
-  } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, a), __builtin_bit_cast(half8v, b), c, 0, 0, 0);
-  }
+__device__ inline void mfma(float4v &c, uint4v a, uint4v b) {
+  if constexpr (BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
+
+// More wait states than any matrix-instruction hazard asks for.
+__device__ inline void settle_matrix_pipe() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 template <bool BF16>
 __device__ inline float widen(uint32_t bits16) {
@@ -85,76 +105,97 @@ __device__ inline uint32_t round_pair(float x0, float x1) {
   return r;
 }
 
-// Writes the 128 x 128 block of results one wavefront holds into the 16-bit C,
-// 16 bytes (8 consecutive rows of one column) per lane and store instruction.
-// The matrix instruction leaves a lane with one row and 16 columns of each
-// 32 x 32 block, so the block is turned through a 32 KiB LDS area that belongs
-// to this wavefront alone: written as fp32 the way the accumulators lie,
-// read back 8 consecutive rows at a time, in two halves of 64 columns.  For an
-// accumulating write the old values are fetched (also 16 bytes per lane)
-// before the LDS pass, added in fp32 and rounded once.  M is a multiple of 8
-// and C is 16-byte aligned (checked by the dispatcher), so a lane's 8 rows are
-// either all inside the matrix or all outside.
+// Writes the R x R block of results one wavefront holds (NBK x NBK blocks of
+// 16 x 16, R = 16 NBK) into the 16-bit C, 16 bytes (8 consecutive rows of one
+// column) per lane and store instruction, R / 8 lanes side by side on a column.
+// The matrix instruction leaves a lane with 4 consecutive rows of one column
+// per block and a wavefront with 16 columns per instruction; stored that way, a
+// store instruction would scatter 32-byte pieces over 16 columns (with a
+// power-of-two leading dimension: 16 requests to one memory channel; measured
+// at twice the time).  So the block is turned through an LDS area that belongs
+// to this wavefront alone, 64 columns (R x 64 floats) at a time: written as
+// fp32, 16 bytes per lane, the way the accumulators lie; read back 8
+// consecutive rows at a time.  For an accumulating write the old values are
+// fetched (also 16 bytes per lane) before the LDS pass, added in fp32 and
+// rounded once.  M is a multiple of 8 and C is 16-byte aligned (checked by the
+// dispatcher), so a lane's 8 rows are either all inside the matrix or all
+// outside.
 //
-// The area holds column c as 128 floats; row r of column c sits at position
-//   r ^ (4 * bit 6 of r) ^ (32 * bit 2 of c).
-// The first term makes the two 16-byte halves of rows 64..127 change places,
-// so that the 16 lanes of one read instruction (8 rows = 32 bytes apart) cover
-// all banks; the second moves the columns the upper half wave writes (4 further
-// on) to the other half of the banks.  Both are constants of a lane's address.
+// The area holds column c as R floats = R / 4 groups of 16 bytes; group G of
+// column c sits at position (G ^ (G >> 4)) ^ (c & 15).  The second term spreads
+// the 16 columns one write instruction touches (and the neighbouring columns
+// one read instruction touches) over all banks; the first swaps the two halves
+// of a lane's 8 rows for rows 64 and up, so that the 16 lanes that read one
+// column of 128 rows cover all banks with their first 16 bytes.  Both are
+// constants of a lane's address up to an XOR with a compile-time value.
 //
-// FULL: the block lies inside the matrix, no lane is masked and the addresses
-// step by a constant; otherwise every access is checked on its own.
-template <bool BF16, bool ACC, bool FULL>
-__device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, int row0, int col0, int lane, int M,
-                                          int N, const float16v (&acc)[4][4]) {
-  const int mc = lane & 15, cq = lane >> 4;
+// FULL: the block lies inside the matrix, no access is masked.
+template <bool BF16, bool ACC, bool FULL, int NBK>
+__device__ inline void emit_blocks_via_lds(unsigned char *area, uint16_t *Cz, long ldc, int row0, int col0, int lane,
+                                           int M, int N, const float4v (&acc)[NBK][NBK]) {
+  constexpr int R = 16 * NBK;      // rows of the block = floats per column of the area
+  constexpr int LPC = R / 8;       // lanes per column on the read side
+  constexpr int CPI = 64 / LPC;    // columns per store instruction
+  constexpr int NIT = 64 / CPI;    // store instructions per pass of 64 columns
+  constexpr int PASSES = R / 64;
+  constexpr int V = 16 / CPI;      // distinct values of (column & 15) / CPI
+  const uint32_t area_addr = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)area;
+
+  // write side: rows 16 i + 4 g .. + 3 of column 16 jl + nl
+  const int g = lane >> 4, nl = lane & 15;
+  uint32_t waddr[NBK];
+#pragma unroll
+  for (int i = 0; i < NBK; ++i) {
+    const int gg = g ^ (i >> 2);  // halves of 8 rows swapped from row 64 on
+    waddr[i] = area_addr + (uint32_t)(nl * R * 4 + 16 * (((4 * i) | gg) ^ nl));
+  }
+  // read side: column CPI it + cq, rows 8 mc .. 8 mc + 7
+  const int mc = lane % LPC, cq = lane / LPC;
   const int m = row0 + 8 * mc;
-  const int flip = mc >> 3;  // rows 64..127: halves swapped
-  // write side: rows 32 i + lane % 32 of columns 32 jl + 8 (v / 4) + 4 (lane / 32) + v % 4
-  float *wbase[4];
+  uint32_t raddr[V];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    wbase[i] = area + (4 * (lane >> 5)) * 128 + ((32 * i + (lane & 31)) ^ (4 * (i >> 1)) ^ (32 * (lane >> 5)));
-  // read side: column 4 it + cq, rows 8 mc .. 8 mc + 7
-  const float *reven = area + cq * 128 + 8 * mc;               // even it
-  const float *rodd = area + cq * 128 + 8 * (mc ^ 4);          // odd it
+  for (int v = 0; v < V; ++v)
+    raddr[v] = area_addr + (uint32_t)(cq * R * 4 + 16 * (((2 * mc) | (mc >> 3)) ^ ((cq + CPI * v) & 15)));
+
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < PASSES; ++h) {
     uint16_t *p0 = Cz + m + (long)(col0 + 64 * h + cq) * ldc;
-    uint32_t ok = 0xffffu;
+    uint32_t ok = ~0u;
     if constexpr (!FULL) {
       ok = 0;
 #pragma unroll
-      for (int it = 0; it < 16; ++it)
-        ok |= (m < M && col0 + 64 * h + 4 * it + cq < N ? 1u : 0u) << it;
+      for (int it = 0; it < NIT; ++it) ok |= (m < M && col0 + 64 * h + CPI * it + cq < N ? 1u : 0u) << it;
     }
     auto live = [&](int it) { return FULL || ((ok >> it) & 1u); };
-    uint4v old[16];
+    uint4v old[NIT];
     if constexpr (ACC) {
 #pragma unroll
-      for (int it = 0; it < 16; ++it) {
+      for (int it = 0; it < NIT; ++it) {
         old[it] = uint4v{0, 0, 0, 0};
-        if (live(it)) old[it] = *reinterpret_cast<const uint4v *>(p0 + (long)(4 * it) * ldc);
+        if (live(it)) old[it] = *reinterpret_cast<const uint4v *>(p0 + (long)(CPI * it) * ldc);
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NBK; ++i)
 #pragma unroll
-      for (int jl = 0; jl < 2; ++jl)
+      for (int jl = 0; jl < 4; ++jl) {
+        // read where the matrix instructions left them: given the choice, the register
+        // allocator moves all accumulators to VGPRs at once and spills
+        float4v x;
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          wbase[i][(32 * jl + 8 * (v / 4) + (v % 4)) * 128] = acc[i][2 * h + jl][v];
-    float4 lo[16], hi[16];
+        for (int v = 0; v < 4; ++v) asm("v_accvgpr_read_b32 %0, %1" : "=v"(x[v]) : "a"(acc[i][4 * h + jl][v]));
+        *(__attribute__((address_space(3))) float4v *)(waddr[i] + (uint32_t)(16 * jl * R * 4)) = x;
+      }
+    float4v lo[NIT], hi[NIT];
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const float4 *src = reinterpret_cast<const float4 *>(((it & 1) ? rodd : reven) + 4 * it * 128);
-      lo[it] = src[flip];
-      hi[it] = src[flip ^ 1];
+    for (int it = 0; it < NIT; ++it) {
+      const uint32_t at = raddr[it % V] + (uint32_t)(CPI * it * R * 4);
+      lo[it] = *(__attribute__((address_space(3))) const float4v *)(at);
+      hi[it] = *(__attribute__((address_space(3))) const float4v *)(at ^ 16u);
     }
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      float f[8] = {lo[it].x, lo[it].y, lo[it].z, lo[it].w, hi[it].x, hi[it].y, hi[it].z, hi[it].w};
+    for (int it = 0; it < NIT; ++it) {
+      float f[8] = {lo[it][0], lo[it][1], lo[it][2], lo[it][3], hi[it][0], hi[it][1], hi[it][2], hi[it][3]};
       uint4v out;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -165,75 +206,8 @@ __device__ inline void emit_block_via_lds(float *area, uint16_t *Cz, long ldc, i
         }
         out[e] = round_pair<BF16>(x0, x1);
       }
-      if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(4 * it) * ldc) = out;
+      if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(CPI * it) * ldc) = out;
     }
-  }
-}
-
-// The same for the 64 x 64 block of a wavefront of the 128 x 128 tiles: one pass
-// through a 16 KiB area of 64 columns x 64 rows.  Row r of column c sits at
-//   r ^ (4 * bit 0 of c) ^ (32 * bit 2 of c):
-// a read instruction covers 8 columns (8 lanes of 8 rows each), and two
-// neighbouring columns, 256 bytes apart, would meet in the same banks without
-// the first term; the second separates the two half waves' writes as above.
-template <bool BF16, bool ACC, bool FULL>
-__device__ inline void emit_block64_via_lds(float *area, uint16_t *Cz, long ldc, int row0, int col0, int lane, int M,
-                                            int N, const float16v (&acc)[2][2]) {
-  const int mc = lane & 7, cq = lane >> 3;
-  const int m = row0 + 8 * mc;
-  const int flip = cq & 1;
-  const int u = lane >> 5, l5 = lane & 31;
-  // write side: rows 32 i + lane % 32 of columns 32 j + 8 (v / 4) + 4 (lane / 32) + v % 4
-  float *wbase[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int par = 0; par < 2; ++par) wbase[i][par] = area + (4 * u) * 64 + 32 * (i ^ u) + (l5 ^ (4 * par));
-  // read side: column 8 it + cq, rows 8 mc .. 8 mc + 7
-  const float *rbase = area + cq * 64 + 8 * (mc ^ (4 * ((cq >> 2) & 1)));
-  uint16_t *p0 = Cz + m + (long)(col0 + cq) * ldc;
-  uint32_t ok = 0xffu;
-  if constexpr (!FULL) {
-    ok = 0;
-#pragma unroll
-    for (int it = 0; it < 8; ++it) ok |= (m < M && col0 + 8 * it + cq < N ? 1u : 0u) << it;
-  }
-  auto live = [&](int it) { return FULL || ((ok >> it) & 1u); };
-  uint4v old[8];
-  if constexpr (ACC) {
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      old[it] = uint4v{0, 0, 0, 0};
-      if (live(it)) old[it] = *reinterpret_cast<const uint4v *>(p0 + (long)(8 * it) * ldc);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) wbase[i][v & 1][(32 * j + 8 * (v / 4) + (v % 4)) * 64] = acc[i][j][v];
-  float4 lo[8], hi[8];
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const float4 *src = reinterpret_cast<const float4 *>(rbase + 8 * it * 64);
-    lo[it] = src[flip];
-    hi[it] = src[flip ^ 1];
-  }
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    float f[8] = {lo[it].x, lo[it].y, lo[it].z, lo[it].w, hi[it].x, hi[it].y, hi[it].z, hi[it].w};
-    uint4v out;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float x0 = f[2 * e], x1 = f[2 * e + 1];
-      if constexpr (ACC) {
-        x0 += widen<BF16>(old[it][e] & 0xffffu);
-        x1 += widen<BF16>(old[it][e] >> 16);
-      }
-      out[e] = round_pair<BF16>(x0, x1);
-    }
-    if (live(it)) *reinterpret_cast<uint4v *>(p0 + (long)(8 * it) * ldc) = out;
   }
 }
 
@@ -250,8 +224,9 @@ __device__ inline void emit_block64_via_lds(float *area, uint16_t *Cz, long ldc,
 //    16 lanes of a 16-byte fragment read (consecutive rows, same c) then hit
 //    16 different 16-byte bank groups.
 //  * m/n-contiguous operand: 64 rows (k) of 256 elements = 512 bytes = 32
-//    chunks.  Chunk c of row k sits at position c ^ ((k & 3) << 2): the four k
-//    rows one transposing read touches land in different bank groups.
+//    chunks.  Chunk c of row k sits at position c ^ ((k & 3) << 2) ^ ((k & 8) >> 2):
+//    the k rows that the lanes of one transposing read touch (four consecutive
+//    ones, and the four 8 further on) land in different bank groups.
 // A load instruction moves 64 x 16 bytes to 1 KiB of consecutive LDS (lane l
 // to byte 16*l), so the swizzle is applied by choosing which global chunk each
 // lane fetches.
@@ -267,92 +242,105 @@ __device__ inline uint4v make_rsrc_words(const uint16_t *p, uint32_t bytes) {
 }
 
 // One 16-byte-per-lane buffer load whose destination is LDS: lane l's data
-// lands at lds_addr + 16*l.  Issued as inline assembly so that the compiler
-// does not put a wait for it in front of every later LDS read; the kernel
-// waits for these loads itself (s_waitcnt vmcnt) before the barrier that
-// publishes the tile.
-__device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+// lands at lds_addr + 16*l and comes from base + voffset + soffset.  Only
+// voffset is checked against the buffer's size, so whatever must read as zero
+// has a voffset past it.  Issued as inline assembly so that the compiler does
+// not put a wait for it in front of every later LDS read; the kernel waits for
+// these loads itself (s_waitcnt vmcnt) before the barrier that publishes the
+// tile.  The wait state between the write of m0 and the load is the one the
+// instruction set asks for.
+__device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
-               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                : "memory");  // m0 is scratch between instructions: nothing else in this kernel keeps a value in it
 }
 
+// The wave's load instructions for one operand: per instruction a lane's byte
+// offset at K tile 0, or kOutOfRange where its row or column lies outside the
+// matrix, and a mask that sends it there in a last K tile that is only partly
+// inside K.
 template <bool KMAJOR, int WB>
 struct LdsLoader {
   static constexpr int NI = 2 * WB;   // the wave's load instructions (1 KiB of LDS each) per operand tile
   static constexpr int CW = 8 * WB;   // (m/n-contiguous) 16-byte chunks per k row of the tile
-  uint32_t off[NI];    // byte offset of this lane's chunk for each of the wave's instructions, at K tile 0
+  uint32_t off[NI];
+  uint32_t cut[NI];    // kOutOfRange where the chunk lies outside a partial last K tile, else 0
   uint32_t step;       // bytes per K tile
-  uint32_t live_mask;  // bit q: instruction q's chunk exists (along the axis that needs a predicate)
-  int kc[NI];          // (k-contiguous only) first k of the chunk inside the tile, per instruction
 
-  __device__ inline void init(long ld, int x0, int X, int wave, int lane) {
-    live_mask = 0;
+  // k_tail: K % BK
+  __device__ inline void init(long ld, int x0, int X, int k_tail, int wave, int lane) {
 #pragma unroll
     for (int q = 0; q < NI; ++q) {
       const int blk = wave * NI + q;  // which 1 KiB block of the region
       if constexpr (KMAJOR) {
         const int x = blk * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((x >> 1) & 7);
-        off[q] = (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2);  // a row past X is past the end
-        kc[q] = c * 8;
+        // a row past X is past the end of the buffer
+        off[q] = (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2);
+        cut[q] = c * 8 < k_tail ? 0u : kOutOfRange;
       } else {
         const int k = blk * (64 / CW) + lane / CW;
-        const int c = (lane % CW) ^ ((k & 3) << 2);
-        off[q] = (uint32_t)(((long)k * ld + x0 + c * 8) * 2);    // a row past K is past the end
-        kc[q] = 0;
-        if (x0 + c * 8 < X) live_mask |= 1u << q;
+        const int c = (lane % CW) ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1);
+        off[q] = x0 + c * 8 < X ? (uint32_t)(((long)k * ld + x0 + c * 8) * 2) : kOutOfRange;
+        cut[q] = k < k_tail ? 0u : kOutOfRange;
       }
     }
     step = KMAJOR ? (uint32_t)(BK * 2) : (uint32_t)(BK * ld * 2);
   }
 
-  // Issues instruction q of K tile `kt_in_r`; `live` false makes it a no-op read.
-  __device__ inline void issue(uint4v rsrc, uint32_t region_addr, int wave, int q, int kt_in_r, int K,
-                               bool live) const {
-    bool in = live;
-    if constexpr (KMAJOR) in = in && kt_in_r * BK + kc[q] < K;
-    else in = in && ((live_mask >> q) & 1u);
-    const uint32_t o = in ? off[q] + (uint32_t)kt_in_r * step : kOutOfRange;
-    lds_dma_b128(rsrc, region_addr + (uint32_t)(wave * NI + q) * 1024u, o);
+  // Issues instruction q for the K tile that starts `soffset` bytes after tile 0;
+  // tail: all ones for a partial last K tile, else 0.
+  __device__ inline void issue(uint4v rsrc, uint32_t region_addr, int wave, int q, uint32_t soffset,
+                               uint32_t tail) const {
+    lds_dma_b128(rsrc, region_addr + (uint32_t)(wave * NI + q) * 1024u, off[q] | (cut[q] & tail), soffset);
   }
 };
 
-// Per-lane constants of the fragment reads of one operand.
+// The LDS addresses of one operand's fragment reads: per-lane values that point
+// into the stage to be read next (`flip` moves them to the other stage), so
+// that every read is one of them plus an immediate.
 template <bool KMAJOR, int WB>
 struct FragReader {
   static constexpr int kPitch = 128 * WB;  // (m/n-contiguous) bytes per k row
-  uint32_t base[4];  // byte offsets inside the region
+  static constexpr int NBK = 2 * WB;       // 16-row blocks of a wavefront's side
+  uint32_t cur[KMAJOR ? 2 : NBK];
 
-  __device__ inline void init(int xw, int lane) {
+  // region_addr: LDS address of the operand's region in stage 0; xw: first row of the wavefront's block
+  __device__ inline void init(uint32_t region_addr, int xw, int lane) {
     if constexpr (KMAJOR) {
-      // row x = xw + 32 i + lane%32, chunk (2 s + lane/32) ^ swizzle: base[s]
-      const int sw = ((lane & 31) >> 1) & 7;
+      // row x = xw + 16 i + lane%16, chunk (4 t + lane/16) ^ swizzle: cur[t]
+      const int sw = ((lane & 15) >> 1) & 7;
 #pragma unroll
-      for (int s = 0; s < 4; ++s)
-        base[s] = (uint32_t)((xw + (lane & 31)) * 128 + (((2 * s + (lane >> 5)) ^ sw) * 16));
+      for (int t = 0; t < 2; ++t)
+        cur[t] = region_addr + (uint32_t)((xw + (lane & 15)) * 128 + (((4 * t + (lane >> 4)) ^ sw) * 16));
     } else {
-      // lane = 16 g + 4 cc + a: supplies k row cc, columns 16 (g%2) + 4 a .. +3: base[i];
-      // chunk xw/8 + 4 i + cl of row k sits at that index ^ (4 (k & 3))
-      const int h = lane >> 5, cc = (lane & 15) >> 2, a = lane & 3;
-      const int cl = (16 * ((lane >> 4) & 1) + 4 * a) >> 3;
+      // lane = 16 g + 4 cc + a supplies k row 8 g + cc (and the one 4 further on),
+      // columns 4 a .. + 3 of the block: cur[i].  Chunk xw/8 + 2 i + a/2 of row k
+      // sits at that index ^ (4 (k & 3)) ^ (2 (k / 8 & 1)) = ^ (4 cc) ^ (2 (g & 1)).
+      const int g = lane >> 4, cc = (lane & 15) >> 2, a = lane & 3;
+      const int sw = (4 * cc) ^ (2 * (g & 1));
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        base[i] = (uint32_t)((8 * h + cc) * kPitch + ((xw / 8 + 4 * i + cl) ^ (4 * cc)) * 16 + (a & 1) * 8);
+      for (int i = 0; i < NBK; ++i)
+        cur[i] = region_addr +
+                 (uint32_t)((8 * g + cc) * kPitch + ((xw / 8 + 2 * i + (a >> 1)) ^ sw) * 16 + (a & 1) * 8);
     }
   }
 
-  // Fragment of 32x32 block i for k step s: 8 consecutive k of row lane%32.
-  __device__ inline uint4v read(const unsigned char *region, int i, int s) const {
+  __device__ inline void flip(uint32_t delta) {
+#pragma unroll
+    for (int e = 0; e < (KMAJOR ? 2 : NBK); ++e) cur[e] += delta;
+  }
+
+  // Fragment of 16-row block i for k step t (32 k): 8 consecutive k, from 8 (lane / 16) on, of row lane % 16.
+  __device__ inline uint4v read(int i, int t) const {
     if constexpr (KMAJOR) {
-      return *reinterpret_cast<const uint4v *>(region + base[s] + i * 4096);
+      return *(__attribute__((address_space(3))) const uint4v *)(cur[t] + (uint32_t)(i * 2048));
     } else {
-      const unsigned char *p = region + base[i] + s * 16 * kPitch;
-      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) short4v *)(p));
+      const uint32_t p = cur[i] + (uint32_t)(t * 32 * kPitch);
+      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(p));
       const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) short4v *)(p + 4 * kPitch));
+          (__attribute__((address_space(3))) short4v *)(p + (uint32_t)(4 * kPitch)));
       uint4v r;
       r.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
       r.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
@@ -370,7 +358,8 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   constexpr int kRegionBytes = kRegion<WB>, kStage2Bytes = kStage<WB>;
   constexpr int WT = 32 * WB;       // rows = columns of a wavefront's block
   constexpr int NI = 2 * WB;        // load instructions per wavefront, operand and K tile
-  constexpr int NB = WB * WB;       // matrix instructions per k step
+  constexpr int NBK = 2 * WB;       // 16 x 16 blocks per side of a wavefront's block
+  constexpr int NB = NBK * NBK;     // matrix instructions per k step of 32
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -390,123 +379,172 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   const int tile_n = in_group / gm;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds2;
+  const int k_tail = g.K % BK;
   LdsLoader<A_KMAJOR, WB> la;
   LdsLoader<B_KMAJOR, WB> lb;
-  la.init(g.lda, m0, g.M, wave, lane);
-  lb.init(g.ldb, n0, g.N, wave, lane);
+  la.init(g.lda, m0, g.M, k_tail, wave, lane);
+  lb.init(g.ldb, n0, g.N, k_tail, wave, lane);
   FragReader<A_KMAJOR, WB> fra;
   FragReader<B_KMAJOR, WB> frb;
-  fra.init(wm * WT, lane);
-  frb.init(wn * WT, lane);
+  fra.init(lds_base, wm * WT, lane);
+  frb.init(lds_base + kRegionBytes, wn * WT, lane);
 
   const uint16_t *Az = g.A + (long)z * g.sA;
   const uint16_t *Bz = g.B + (long)z * g.sB;
 
-  float16v acc[WB][WB];
+  float4v acc[NBK][NBK];
 #pragma unroll
-  for (int i = 0; i < WB; ++i)
+  for (int i = 0; i < NBK; ++i)
 #pragma unroll
-    for (int j = 0; j < WB; ++j)
+    for (int j = 0; j < NBK; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
 
   const int kt_end = g.total_ktiles;
   // Every workgroup starts its walk over K at a different tile (and wraps
   // around): with power-of-two leading dimensions, workgroups marching through
   // K in lockstep would all pull from the same memory channels at once.
-  const int kt_rot = (tile_m + tile_n + z) % kt_end;
-  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds2;
-  auto issue_tile = [&](int kt, int q_first, int q_count) {
-    // instructions [q_first, q_first + q_count) of the 2 NI that move K tile kt (NI for A, then NI for B)
-    const bool live = kt < kt_end;
-    int ktc = live ? kt + kt_rot : 0;
-    ktc = ktc >= kt_end ? ktc - kt_end : ktc;
-    const int r = ktc / g.ktiles_per_r;
-    const int kt_in_r = ktc - r * g.ktiles_per_r;
-    const uint32_t stage = lds_base + (uint32_t)(kt & 1) * kStage2Bytes;
-#pragma unroll
-    for (int q = q_first; q < q_first + q_count; ++q) {
-      if (q < NI) la.issue(make_rsrc_words(Az + (long)r * g.rA, g.a_bytes), stage, wave, q, kt_in_r, g.K, live);
-      else lb.issue(make_rsrc_words(Bz + (long)r * g.rB, g.b_bytes), stage + kRegionBytes, wave, q - NI, kt_in_r,
-                    g.K, live);
+  //
+  // State of the K tile to be loaded next, all scalar: which K range (r) and
+  // which tile inside it, advanced by one tile at a time.
+  int ld_ktc = (tile_m + tile_n + z) % kt_end;
+  int ld_r = ld_ktc / g.ktiles_per_r;
+  int ld_kin = ld_ktc - ld_r * g.ktiles_per_r;
+  uint4v rs_a, rs_b;        // buffer descriptors of the K range
+  uint32_t so_a, so_b;      // byte offset of the tile inside it
+  uint32_t ld_tail;         // all ones: the tile is only partly inside K
+  auto describe_range = [&]() {
+    rs_a = make_rsrc_words(Az + (long)ld_r * g.rA, g.a_bytes);
+    rs_b = make_rsrc_words(Bz + (long)ld_r * g.rB, g.b_bytes);
+  };
+  auto describe_tile = [&]() {
+    so_a = (uint32_t)ld_kin * la.step;
+    so_b = (uint32_t)ld_kin * lb.step;
+    ld_tail = (uint32_t)__builtin_amdgcn_readfirstlane(k_tail != 0 && ld_kin == g.ktiles_per_r - 1 ? -1 : 0);
+  };
+  auto next_tile = [&]() {
+    ++ld_ktc;
+    ++ld_kin;
+    if (ld_kin == g.ktiles_per_r) {
+      ld_kin = 0;
+      ++ld_r;
     }
+    if (ld_ktc == kt_end) ld_ktc = ld_r = ld_kin = 0;
+  };
+  // instruction q of the 2 NI that move the described tile into `stage` (NI for A, then NI for B)
+  auto issue = [&](int q, int stage) {
+    const uint32_t st = lds_base + (uint32_t)stage * kStage2Bytes;
+    if (q < NI) la.issue(rs_a, st, wave, q, so_a, ld_tail);
+    else lb.issue(rs_b, st + kRegionBytes, wave, q - NI, so_b, ld_tail);
   };
 
-  issue_tile(0, 0, 2 * NI);
-  issue_tile(1, 0, 2 * NI);
-  // tile 0 has landed once all but the newest 2 NI loads are done
-  if constexpr (WB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  describe_range();
+  describe_tile();
+#pragma unroll
+  for (int q = 0; q < 2 * NI; ++q) issue(q, 0);
+  if (kt_end > 1) {
+    next_tile();
+    describe_range();
+    describe_tile();
+#pragma unroll
+    for (int q = 0; q < 2 * NI; ++q) issue(q, 1);
+  }
+  // tile 0 has landed once all but the newest 2 NI loads (if tile 1 exists) are done
+  if (kt_end > 1) {
+    if constexpr (WB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
 
-  // Fragments of the four k steps of a tile live in four register buffers and
-  // are read two steps ahead: steps 2 and 3 of this tile during steps 0 and 1,
-  // then - behind the barrier - steps 0 and 1 of the next tile during steps 2
-  // and 3.  The barrier therefore sits in the middle of a tile, and the
+  // The fragments of the two k steps of a tile live in two register buffers and
+  // are read one step (NB matrix instructions) ahead: step 1 of this tile
+  // during step 0, then - behind the barrier - step 0 of the next tile during
+  // step 1.  The barrier therefore sits in the middle of a tile, and the
   // global-to-LDS loads that refill the stage (K tile kt+2) are spread over
-  // the instruction slots of steps 2 and 3, with a whole tile time to land.
-  uint4v fa[4][WB], fb[4][WB];
-  auto read_frag = [&](int buf, int q, int stage, int s) {
-    const unsigned char *st = lds2 + stage * kStage2Bytes;
-    if (q < WB) fa[buf][q] = fra.read(st, q, s);
-    else fb[buf][q - WB] = frb.read(st + kRegionBytes, q - WB, s);
+  // the instruction slots of step 1, with a whole tile time to land.
+  //
+  // A matrix instruction keeps its pipe busy for 16 cycles and the wavefront
+  // issues one instruction every 4: whatever sits between two of them must be
+  // at most three instructions, or the pipe idles.  Hence the scalar
+  // bookkeeping of the next load is dealt out over the free slots of step 0
+  // (pinned there by empty asm statements), a load costs four instructions
+  // (select, m0, wait state, load), and every LDS address is a register plus
+  // an immediate.
+  uint4v fa[2][NBK], fb[2][NBK];
+  auto read_frag = [&](int buf, int q, int t) {
+    if (q < NBK) fa[buf][q] = fra.read(q, t);
+    else fb[buf][q - NBK] = frb.read(q - NBK, t);
   };
 #pragma unroll
-  for (int q = 0; q < 2 * WB; ++q) read_frag(0, q, 0, 0);
-#pragma unroll
-  for (int q = 0; q < 2 * WB; ++q) read_frag(1, q, 0, 1);
+  for (int q = 0; q < 2 * NBK; ++q) read_frag(0, q, 0);
 
-  // the 2 NI loads of a K tile go out in steps 2 and 3: NI per step, one every NB / NI matrix instructions
-  constexpr int kEvery = NB / NI;
-  for (int kt = 0; kt < kt_end; ++kt) {
+  // the 2 NI loads of a K tile go out in step 1, one every NB / (2 NI) matrix instructions
+  constexpr int kEvery = NB / (2 * NI);
+  uint32_t flip_by = (uint32_t)kStage2Bytes;  // to the other stage and back
+  settle_matrix_pipe();  // the zeroed accumulators
+  // one K tile; LOADS: K tile kt + 2 exists and is fetched
+  auto tile = [&](auto loads_tag, int kt) {
+    constexpr bool loads = decltype(loads_tag)::value;
     const int stage = kt & 1;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int t = 0; t < 2; ++t) {
 #pragma unroll
       for (int q = 0; q < NB; ++q) {
-        const int i = q / WB, j = q % WB;
-        acc[i][j] = mfma<BF16>(fb[s][j], fa[s][i], acc[i][j]);
-        if (q < 2 * WB) {
-          if (s < 2) read_frag(s + 2, q, stage, s + 2);
-          else read_frag(s - 2, q, stage ^ 1, s - 2);
+        const int i = q / NBK, j = q % NBK;
+        mfma<BF16>(acc[i][j], fa[t][i], fb[t][j]);
+        if (q < 2 * NBK) read_frag(t ^ 1, q, t ^ 1);
+        if constexpr (loads) {
+          if (t == 0) {
+            // the tile after the one in flight: described piece by piece
+            if (q == 2 * NBK) {
+              next_tile();
+              asm volatile("" : "+s"(ld_ktc), "+s"(ld_r), "+s"(ld_kin));
+            } else if (q == 2 * NBK + 2) {
+              if (g.ktiles_per_r != kt_end) describe_range();
+              asm volatile("" : "+s"(rs_a), "+s"(rs_b));
+            } else if (q == 2 * NBK + 4) {
+              describe_tile();
+              asm volatile("" : "+s"(so_a), "+s"(so_b), "+s"(ld_tail));
+            }
+          } else if (q % kEvery == kEvery - 1) {
+            issue(q / kEvery, stage);
+          }
         }
-        if (s >= 2 && q % kEvery == kEvery - 1) issue_tile(kt + 2, (s - 2) * NI + q / kEvery, 1);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 1) {
+      if (t == 0) {
         // own loads of tile kt+1 have landed, own reads of this stage are done;
         // behind the barrier that holds for every wave
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
+        fra.flip(flip_by);
+        frb.flip(flip_by);
+        flip_by = 0u - flip_by;
       }
     }
-  }
-  // The loads issued for tiles past the end move nothing, but must have retired,
-  // and every wave must be done with the stages, before LDS is reused below.
+  };
+  int kt = 0;
+  for (; kt + 2 < kt_end; ++kt) tile(std::true_type{}, kt);
+  for (; kt < kt_end; ++kt) tile(std::false_type{}, kt);
+  // every wave must be done with the stages before LDS is reused below
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
+  settle_matrix_pipe();
 
   uint16_t *Cz = g.C + (long)z * g.sC;
   const int row0 = m0 + wm * WT, col0 = n0 + wn * WT;
   const bool full = row0 + WT <= g.M && col0 + WT <= g.N;  // the same for every lane of the wavefront
-  if constexpr (WB == 4) {
-    float *area = reinterpret_cast<float *>(lds2 + wave * kRegionBytes);
-    if (g.accumulate) {
-      if (full) emit_block_via_lds<BF16, true, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-      else emit_block_via_lds<BF16, true, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-    } else {
-      if (full) emit_block_via_lds<BF16, false, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-      else emit_block_via_lds<BF16, false, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-    }
+  // the stage buffers are free by now: a quarter of them per wavefront
+  unsigned char *area = lds2 + wave * (kLds<WB> / 4);
+  if (g.accumulate) {
+    if (full) emit_blocks_via_lds<BF16, true, true, NBK>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+    else emit_blocks_via_lds<BF16, true, false, NBK>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
   } else {
-    float *area = reinterpret_cast<float *>(lds2 + wave * (kLds<WB> / 4));
-    if (g.accumulate) {
-      if (full) emit_block64_via_lds<BF16, true, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-      else emit_block64_via_lds<BF16, true, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-    } else {
-      if (full) emit_block64_via_lds<BF16, false, true>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-      else emit_block64_via_lds<BF16, false, false>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
-    }
+    if (full) emit_blocks_via_lds<BF16, false, true, NBK>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
+    else emit_blocks_via_lds<BF16, false, false, NBK>(area, Cz, g.ldc, row0, col0, lane, g.M, g.N, acc);
   }
 }
 
