@@ -41,9 +41,11 @@ __device__ inline uint4v make_rsrc_words(const float *p, uint32_t bytes) {
 // lands at lds_addr + 16*l.  Inline assembly keeps the compiler from putting a
 // wait for it in front of every later LDS read; the kernel waits for these
 // loads itself (s_waitcnt vmcnt) before the barrier that publishes the tile.
-// m0 is scratch between instructions: nothing else here keeps a value in it.
+// m0 is scratch between instructions: nothing else here keeps a value in it;
+// the wait state between its write and the load is the one the instruction set
+// asks for.
 __device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                :
                : "s"(lds_addr), "v"(voffset), "s"(rsrc)
                : "memory");
@@ -51,7 +53,7 @@ __device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t vof
 
 // The 4-byte form: lane l's data lands at lds_addr + 4*l.
 __device__ inline void lds_dma_b32(uint4v rsrc, uint32_t lds_addr, uint32_t voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
                :
                : "s"(lds_addr), "v"(voffset), "s"(rsrc)
                : "memory");

@@ -327,9 +327,17 @@ struct FragReader {
     }
   }
 
-  __device__ inline void flip(uint32_t delta) {
-#pragma unroll
-    for (int e = 0; e < (KMAJOR ? 2 : NBK); ++e) cur[e] += delta;
+  // Moves the addresses that block i's reads use to the other stage; called for
+  // every block in turn, just before its first read from that stage.
+  __device__ inline void flip(int i, uint32_t delta) {
+    if constexpr (KMAJOR) {
+      if (i == 0) {
+        cur[0] += delta;
+        cur[1] += delta;
+      }
+    } else {
+      cur[i] += delta;
+    }
   }
 
   // Fragment of 16-row block i for k step t (32 k): 8 consecutive k, from 8 (lane / 16) on, of row lane % 16.
@@ -481,8 +489,9 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
 #pragma unroll
   for (int q = 0; q < 2 * NBK; ++q) read_frag(0, q, 0);
 
-  // the 2 NI loads of a K tile go out in step 1, one every NB / (2 NI) matrix instructions
-  constexpr int kEvery = NB / (2 * NI);
+  // the 2 NI loads of a K tile go out in step 1, in the slots behind the fragment reads
+  constexpr int kEvery = (NB - 2 * NBK) / (2 * NI);
+  static_assert(kEvery >= 1 && kEvery * 2 * NI == NB - 2 * NBK, "one load every kEvery slots fills step 1");
   uint32_t flip_by = (uint32_t)kStage2Bytes;  // to the other stage and back
   settle_matrix_pipe();  // the zeroed accumulators
   // one K tile; LOADS: K tile kt + 2 exists and is fetched
@@ -495,22 +504,37 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
       for (int q = 0; q < NB; ++q) {
         const int i = q / NBK, j = q % NBK;
         mfma<BF16>(acc[i][j], fa[t][i], fb[t][j]);
-        if (q < 2 * NBK) read_frag(t ^ 1, q, t ^ 1);
+        if (q < 2 * NBK) {
+          if (t == 1) {
+            // behind the barrier: on to the other stage
+            if (q < NBK) fra.flip(q, flip_by);
+            else frb.flip(q - NBK, flip_by);
+          }
+          read_frag(t ^ 1, q, t ^ 1);
+        }
         if constexpr (loads) {
           if (t == 0) {
             // the tile after the one in flight: described piece by piece
             if (q == 2 * NBK) {
-              next_tile();
+              ++ld_ktc;
+              ++ld_kin;
+              if (ld_kin == g.ktiles_per_r) {
+                ld_kin = 0;
+                ++ld_r;
+              }
               asm volatile("" : "+s"(ld_ktc), "+s"(ld_r), "+s"(ld_kin));
             } else if (q == 2 * NBK + 2) {
+              if (ld_ktc == kt_end) ld_ktc = ld_r = ld_kin = 0;
+              asm volatile("" : "+s"(ld_ktc), "+s"(ld_r), "+s"(ld_kin));
+            } else if (q == 2 * NBK + 4) {
               if (g.ktiles_per_r != kt_end) describe_range();
               asm volatile("" : "+s"(rs_a), "+s"(rs_b));
-            } else if (q == 2 * NBK + 4) {
+            } else if (q == 2 * NBK + 6) {
               describe_tile();
               asm volatile("" : "+s"(so_a), "+s"(so_b), "+s"(ld_tail));
             }
-          } else if (q % kEvery == kEvery - 1) {
-            issue(q / kEvery, stage);
+          } else if (q >= 2 * NBK && (q - 2 * NBK) % kEvery == kEvery - 1) {
+            issue((q - 2 * NBK) / kEvery, stage);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -520,8 +544,7 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
         // behind the barrier that holds for every wave
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
-        fra.flip(flip_by);
-        frb.flip(flip_by);
+      } else {
         flip_by = 0u - flip_by;
       }
     }
