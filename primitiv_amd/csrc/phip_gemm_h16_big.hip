@@ -242,18 +242,19 @@ __device__ inline uint4v make_rsrc_words(const uint16_t *p, uint32_t bytes) {
 }
 
 // One 16-byte-per-lane buffer load whose destination is LDS: lane l's data
-// lands at lds_addr + 16*l and comes from base + voffset + soffset.  Only
-// voffset is checked against the buffer's size, so whatever must read as zero
-// has a voffset past it.  Issued as inline assembly so that the compiler does
-// not put a wait for it in front of every later LDS read; the kernel waits for
-// these loads itself (s_waitcnt vmcnt) before the barrier that publishes the
-// tile.  The wait state between the write of m0 and the load is the one the
-// instruction set asks for.
-__device__ inline void lds_dma_b128(uint4v rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
-               : "memory");  // m0 is scratch between instructions: nothing else in this kernel keeps a value in it
+// lands at lds_addr + 16*l and comes from base + voffset + soffset; lds_addr
+// then moves on by the 1 KiB the load fills.  Only voffset is checked against
+// the buffer's size, so whatever must read as zero has a voffset past it.
+// Issued as inline assembly so that the compiler does not put a wait for it in
+// front of every later LDS read; the kernel waits for these loads itself
+// (s_waitcnt vmcnt) before the barrier that publishes the tile.  The
+// instruction set asks for a wait state between the write of m0 and the load:
+// the addition sits there.
+__device__ inline void lds_dma_b128(uint4v rsrc, uint32_t &lds_addr, uint32_t voffset, uint32_t soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_add_u32 %0, %0, 0x400\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               : "+s"(lds_addr)
+               : "v"(voffset), "s"(rsrc), "s"(soffset)
+               : "memory", "scc");  // m0 is scratch between instructions: nothing else in this kernel keeps a value in it
 }
 
 // The wave's load instructions for one operand: per instruction a lane's byte
@@ -266,6 +267,7 @@ struct LdsLoader {
   static constexpr int CW = 8 * WB;   // (m/n-contiguous) 16-byte chunks per k row of the tile
   uint32_t off[NI];
   uint32_t cut[NI];    // kOutOfRange where the chunk lies outside a partial last K tile, else 0
+  uint32_t use[NI];    // what the loads take: off, or off | cut while a partial tile is being fetched
   uint32_t step;       // bytes per K tile
 
   // k_tail: K % BK
@@ -287,13 +289,19 @@ struct LdsLoader {
       }
     }
     step = KMAJOR ? (uint32_t)(BK * 2) : (uint32_t)(BK * ld * 2);
+    select(0u);
   }
 
-  // Issues instruction q for the K tile that starts `soffset` bytes after tile 0;
-  // tail: all ones for a partial last K tile, else 0.
-  __device__ inline void issue(uint4v rsrc, uint32_t region_addr, int wave, int q, uint32_t soffset,
-                               uint32_t tail) const {
-    lds_dma_b128(rsrc, region_addr + (uint32_t)(wave * NI + q) * 1024u, off[q] | (cut[q] & tail), soffset);
+  // tail: all ones before the loads of a partial last K tile, 0 before those of a whole one
+  __device__ inline void select(uint32_t tail) {
+#pragma unroll
+    for (int q = 0; q < NI; ++q) use[q] = off[q] | (cut[q] & tail);
+  }
+
+  // Issues instruction q for the K tile that starts `soffset` bytes after tile 0
+  // into the next 1 KiB at lds_addr.
+  __device__ inline void issue(uint4v rsrc, uint32_t &lds_addr, int q, uint32_t soffset) const {
+    lds_dma_b128(rsrc, lds_addr, use[q], soffset);
   }
 };
 
@@ -422,6 +430,8 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   uint4v rs_a, rs_b;        // buffer descriptors of the K range
   uint32_t so_a, so_b;      // byte offset of the tile inside it
   uint32_t ld_tail;         // all ones: the tile is only partly inside K
+  uint32_t sel_tail = 0;    // what the loaders' offsets are selected for
+  uint32_t lds_run = 0;     // LDS address of the next load
   auto describe_range = [&]() {
     rs_a = make_rsrc_words(Az + (long)ld_r * g.rA, g.a_bytes);
     rs_b = make_rsrc_words(Bz + (long)ld_r * g.rB, g.b_bytes);
@@ -440,21 +450,33 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
     }
     if (ld_ktc == kt_end) ld_ktc = ld_r = ld_kin = 0;
   };
-  // instruction q of the 2 NI that move the described tile into `stage` (NI for A, then NI for B)
+  // a partial tile comes up, or is over (twice per K range at most)
+  auto select_offsets = [&]() {
+    if (ld_tail != sel_tail) {
+      la.select(ld_tail);
+      lb.select(ld_tail);
+      sel_tail = ld_tail;
+    }
+  };
+  // instruction q of the 2 NI that move the described tile into `stage` (NI for A, then NI for B):
+  // the wave's share of each region is NI consecutive KiB
   auto issue = [&](int q, int stage) {
-    const uint32_t st = lds_base + (uint32_t)stage * kStage2Bytes;
-    if (q < NI) la.issue(rs_a, st, wave, q, so_a, ld_tail);
-    else lb.issue(rs_b, st + kRegionBytes, wave, q - NI, so_b, ld_tail);
+    if (q == 0) lds_run = lds_base + (uint32_t)stage * kStage2Bytes + (uint32_t)(wave * NI) * 1024u;
+    if (q == NI) lds_run += (uint32_t)(kRegionBytes - NI * 1024);
+    if (q < NI) la.issue(rs_a, lds_run, q, so_a);
+    else lb.issue(rs_b, lds_run, q - NI, so_b);
   };
 
   describe_range();
   describe_tile();
+  select_offsets();
 #pragma unroll
   for (int q = 0; q < 2 * NI; ++q) issue(q, 0);
   if (kt_end > 1) {
     next_tile();
     describe_range();
     describe_tile();
+    select_offsets();
 #pragma unroll
     for (int q = 0; q < 2 * NI; ++q) issue(q, 1);
   }
@@ -478,9 +500,9 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   // issues one instruction every 4: whatever sits between two of them must be
   // at most three instructions, or the pipe idles.  Hence the scalar
   // bookkeeping of the next load is dealt out over the free slots of step 0
-  // (pinned there by empty asm statements), a load costs four instructions
-  // (select, m0, wait state, load), and every LDS address is a register plus
-  // an immediate.
+  // (pinned there by empty asm statements), a load costs three instructions
+  // (m0, the next LDS address, the load), and every LDS address is a register
+  // plus an immediate.
   uint4v fa[2][NBK], fb[2][NBK];
   auto read_frag = [&](int buf, int q, int t) {
     if (q < NBK) fa[buf][q] = fra.read(q, t);
@@ -532,6 +554,8 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
             } else if (q == 2 * NBK + 6) {
               describe_tile();
               asm volatile("" : "+s"(so_a), "+s"(so_b), "+s"(ld_tail));
+            } else if (q == 2 * NBK + 7) {
+              select_offsets();
             }
           } else if (q >= 2 * NBK && (q - 2 * NBK) % kEvery == kEvery - 1) {
             issue((q - 2 * NBK) / kEvery, stage);
