@@ -511,7 +511,7 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
 #pragma unroll
   for (int q = 0; q < 2 * NBK; ++q) read_frag(0, q, 0);
 
-  // the 2 NI loads of a K tile go out in step 1, in the slots behind the fragment reads
+  // the 2 NI loads of a K tile go out in step 1; in the large tiles in the slots behind the fragment reads
   constexpr int kEvery = (NB - 2 * NBK) / (2 * NI);
   static_assert(kEvery >= 1 && kEvery * 2 * NI == NB - 2 * NBK, "one load every kEvery slots fills step 1");
   uint32_t flip_by = (uint32_t)kStage2Bytes;  // to the other stage and back
@@ -557,8 +557,11 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
             } else if (q == 2 * NBK + 7) {
               select_offsets();
             }
-          } else if (q >= 2 * NBK && (q - 2 * NBK) % kEvery == kEvery - 1) {
-            issue((q - 2 * NBK) / kEvery, stage);
+          } else if constexpr (WB == 4) {
+            if (q >= 2 * NBK && (q - 2 * NBK) % kEvery == kEvery - 1) issue((q - 2 * NBK) / kEvery, stage);
+          } else {
+            // few matrix instructions per tile: the loop waits for these loads, so out they go at once
+            if (q < 2 * NI) issue(q, stage);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
