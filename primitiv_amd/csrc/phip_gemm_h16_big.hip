@@ -37,6 +37,12 @@ typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
+// LDS pointer from an LDS byte address (a register plus an immediate, for the compiler)
+template <class T>
+__device__ inline __attribute__((address_space(3))) T *lds_ptr(uint32_t addr) {
+  return (__attribute__((address_space(3))) T *)(size_t)addr;
+}
+
 constexpr int kThreads = 256;
 constexpr int BK = 64;
 // WB = 32 rows (two blocks of 16) per wavefront and direction: 4 -> 256 x 256 tiles (one workgroup per
@@ -184,14 +190,14 @@ __device__ inline void emit_blocks_via_lds(unsigned char *area, uint16_t *Cz, lo
         float4v x;
 #pragma unroll
         for (int v = 0; v < 4; ++v) asm("v_accvgpr_read_b32 %0, %1" : "=v"(x[v]) : "a"(acc[i][4 * h + jl][v]));
-        *(__attribute__((address_space(3))) float4v *)(waddr[i] + (uint32_t)(16 * jl * R * 4)) = x;
+        *lds_ptr<float4v>(waddr[i] + (uint32_t)(16 * jl * R * 4)) = x;
       }
     float4v lo[NIT], hi[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const uint32_t at = raddr[it % V] + (uint32_t)(CPI * it * R * 4);
-      lo[it] = *(__attribute__((address_space(3))) const float4v *)(at);
-      hi[it] = *(__attribute__((address_space(3))) const float4v *)(at ^ 16u);
+      lo[it] = *lds_ptr<const float4v>(at);
+      hi[it] = *lds_ptr<const float4v>(at ^ 16u);
     }
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
@@ -351,12 +357,11 @@ struct FragReader {
   // Fragment of 16-row block i for k step t (32 k): 8 consecutive k, from 8 (lane / 16) on, of row lane % 16.
   __device__ inline uint4v read(int i, int t) const {
     if constexpr (KMAJOR) {
-      return *(__attribute__((address_space(3))) const uint4v *)(cur[t] + (uint32_t)(i * 2048));
+      return *lds_ptr<const uint4v>(cur[t] + (uint32_t)(i * 2048));
     } else {
       const uint32_t p = cur[i] + (uint32_t)(t * 32 * kPitch);
-      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(p));
-      const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) short4v *)(p + (uint32_t)(4 * kPitch)));
+      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(lds_ptr<short4v>(p));
+      const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(lds_ptr<short4v>(p + (uint32_t)(4 * kPitch)));
       uint4v r;
       r.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
       r.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
@@ -511,9 +516,7 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
 #pragma unroll
   for (int q = 0; q < 2 * NBK; ++q) read_frag(0, q, 0);
 
-  // the 2 NI loads of a K tile go out in step 1; in the large tiles in the slots behind the fragment reads
-  constexpr int kEvery = (NB - 2 * NBK) / (2 * NI);
-  static_assert(kEvery >= 1 && kEvery * 2 * NI == NB - 2 * NBK, "one load every kEvery slots fills step 1");
+  static_assert(WB == 2 || NB >= 3 * 2 * NBK, "every third slot holds a read");
   uint32_t flip_by = (uint32_t)kStage2Bytes;  // to the other stage and back
   settle_matrix_pipe();  // the zeroed accumulators
   // one K tile; LOADS: K tile kt + 2 exists and is fetched
@@ -526,18 +529,27 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
       for (int q = 0; q < NB; ++q) {
         const int i = q / NBK, j = q % NBK;
         mfma<BF16>(acc[i][j], fa[t][i], fb[t][j]);
-        if (q < 2 * NBK) {
+        // Slot plan.  Large tiles: the 4 waves' reads of a step are 64 KiB, 512 cycles
+        // of LDS time, so one read per slot (16 cycles) asks for twice what LDS
+        // delivers and the reads queue up in front of the matrix instructions;
+        // one every third slot does not.  The loads take the slots after them,
+        // the bookkeeping the third kind.  Small tiles: reads, then the rest.
+        constexpr int kSpread = WB == 4 ? 3 : 1;
+        const int rq = q / kSpread;  // which read / load / piece of bookkeeping
+        const int kind = WB == 4 ? q % kSpread : (q < 2 * NBK ? 0 : 2);
+        if (kind == 0 && rq < 2 * NBK) {
           if (t == 1) {
             // behind the barrier: on to the other stage
-            if (q < NBK) fra.flip(q, flip_by);
-            else frb.flip(q - NBK, flip_by);
+            if (rq < NBK) fra.flip(rq, flip_by);
+            else frb.flip(rq - NBK, flip_by);
           }
-          read_frag(t ^ 1, q, t ^ 1);
+          read_frag(t ^ 1, rq, t ^ 1);
         }
         if constexpr (loads) {
           if (t == 0) {
             // the tile after the one in flight: described piece by piece
-            if (q == 2 * NBK) {
+            const int piece = WB == 4 ? (kind == 2 ? rq : -1) : q - 2 * NBK;
+            if (piece == 0) {
               ++ld_ktc;
               ++ld_kin;
               if (ld_kin == g.ktiles_per_r) {
@@ -545,20 +557,20 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
                 ++ld_r;
               }
               asm volatile("" : "+s"(ld_ktc), "+s"(ld_r), "+s"(ld_kin));
-            } else if (q == 2 * NBK + 2) {
+            } else if (piece == 2) {
               if (ld_ktc == kt_end) ld_ktc = ld_r = ld_kin = 0;
               asm volatile("" : "+s"(ld_ktc), "+s"(ld_r), "+s"(ld_kin));
-            } else if (q == 2 * NBK + 4) {
+            } else if (piece == 4) {
               if (g.ktiles_per_r != kt_end) describe_range();
               asm volatile("" : "+s"(rs_a), "+s"(rs_b));
-            } else if (q == 2 * NBK + 6) {
+            } else if (piece == 6) {
               describe_tile();
               asm volatile("" : "+s"(so_a), "+s"(so_b), "+s"(ld_tail));
-            } else if (q == 2 * NBK + 7) {
+            } else if (piece == 7) {
               select_offsets();
             }
           } else if constexpr (WB == 4) {
-            if (q >= 2 * NBK && (q - 2 * NBK) % kEvery == kEvery - 1) issue((q - 2 * NBK) / kEvery, stage);
+            if (kind == 1 && rq < 2 * NI) issue(rq, stage);
           } else {
             // few matrix instructions per tile: the loop waits for these loads, so out they go at once
             if (q < 2 * NI) issue(q, stage);
