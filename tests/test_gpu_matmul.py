@@ -412,6 +412,9 @@ BIG_H16 = [  # di, dj, dk, ba, bb
     (776, 520, 1032, 16, 16),
     (136, 2824, 2832, 16, 1),
     (2824, 264, 712, 1, 4),
+    # one partial K tile, and two K tiles of which the second is partial, in the forward product
+    (4096, 24, 4096, 1, 1),
+    (3080, 72, 3592, 1, 1),
     # too few 256 x 256 tiles for the chip: 128 x 128 tiles, all three products / per-sample / shared a
     (1480, 1608, 1544, 1, 1),
     (520, 392, 264, 12, 12),
