@@ -78,7 +78,7 @@ struct DmaLoader {
       if constexpr (KMAJOR) {
         const int x = blk * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((x >> 1) & 7);
-        off[q] = (uint32_t)(((long)(x0 + x) * ld + c * 4) * 4);  // a row past X is past the end
+        off[q] = x0 + x < X ? (uint32_t)(((long)(x0 + x) * ld + c * 4) * 4) : kOutOfRange;
         kc[q] = c * 4;
       } else {
         const int k = blk * (64 / kLanesPerRow) + lane / kLanesPerRow;

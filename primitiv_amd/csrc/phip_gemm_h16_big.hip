@@ -284,8 +284,7 @@ struct LdsLoader {
       if constexpr (KMAJOR) {
         const int x = blk * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((x >> 1) & 7);
-        // a row past X is past the end of the buffer
-        off[q] = (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2);
+        off[q] = x0 + x < X ? (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2) : kOutOfRange;
         cut[q] = c * 8 < k_tail ? 0u : kOutOfRange;
       } else {
         const int k = blk * (64 / CW) + lane / CW;
