@@ -56,6 +56,31 @@ static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, voi
     g.N = (int)(dk * bb);
     g.batch = 1;
   }
+  // 16-bit storage, one large a against many columns: the large-tile kernel runs
+  // at the power limit there, and its K loop settles at a clock a sixth higher
+  // when both operands are contiguous along k (16-byte LDS reads) than when a
+  // is transposed by the LDS reads (1.49 against 1.28 GHz, fp16, counted in the
+  // kernel).  A transposed copy of a costs one pass over it; from 16 Ki columns
+  // on that is less than what the product gains.
+  if (elem != Elem::F32 && ba == 1 && di >= 1024 && dj >= 1024 && di % 8 == 0 && dj % 8 == 0 &&
+      (long)dk * bb >= 16384 && (long)di * dj * 2 < (1L << 31)) {
+    struct Block {  // back to the pool on every way out; the stream orders its reuse
+      phip_ctx *ctx;
+      void *ptr;
+      ~Block() {
+        if (ptr) phip_pool_free(ctx, ptr);
+      }
+    } at{ctx, nullptr};
+    rc = phip_pool_alloc(ctx, (size_t)di * dj * 2, &at.ptr, nullptr);
+    if (rc != PHIP_OK) return rc;
+    rc = elem == Elem::F16 ? phip_transpose_fw_f16(ctx, a, at.ptr, di, dj, 1)
+                           : phip_transpose_fw_bf16(ctx, a, at.ptr, di, dj, 1);
+    if (rc != PHIP_OK) return rc;
+    g.A = at.ptr;      // a^T: element (m, k) at k + m*dj
+    g.lda = dj;
+    g.a_kmajor = true;
+    return gemm_dispatch(ctx, g, elem);
+  }
   return gemm_dispatch(ctx, g, elem);
 }
 
