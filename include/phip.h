@@ -158,6 +158,23 @@ int phip_matmul_fw_f16(phip_ctx *ctx, const void *a, const void *b, void *y,
 int phip_matmul_fw_bf16(phip_ctx *ctx, const void *a, const void *b, void *y,
                         uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
 
+/* ---- matmul forward without any allocation ---------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device
+ * memory during the call: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments, kernels and result bits as
+ * phip_matmul_fw_f32; a product whose K range is split between workgroups
+ * keeps its partial tiles and tile counters in a fixed array inside the
+ * library's device code (PHIP_NOALLOC_SCRATCH_BYTES per GPU, held until the
+ * process ends) instead of a pool block.  Calls no hipMalloc / hipFree and
+ * leaves the context's pool untouched.  A product that needs more scratch than
+ * the array holds fails with PHIP_ERR_INVALID_ARGUMENT before anything has
+ * been written to y.  All contexts on one GPU share that GPU's array: calls of
+ * this entry point that overlap on one GPU (two contexts, i.e. two streams)
+ * race; calls on one context are ordered by its stream. */
+#define PHIP_NOALLOC_SCRATCH_BYTES (16u << 20)
+int phip_matmul_fw_f32_noalloc(phip_ctx *ctx, const float *a, const float *b, float *y,
+                               uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
+
 /* ---- matmul backward:  ga += gy . b^T ,  gb += a^T . gy --------------------
  * Reference: Device::matmul_bw_impl (primitiv/core/device.h:481-483;
  * primitiv/devices/eigen/ops/matmul.cc:40-79; primitiv/devices/cuda/ops/matmul.cu:

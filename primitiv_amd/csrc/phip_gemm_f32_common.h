@@ -211,7 +211,7 @@ struct Scratch {
   void *ptr = nullptr;
   explicit Scratch(phip_ctx *c) : ctx(c) {}
   ~Scratch() {
-    if (ptr) phip_pool_free(ctx, ptr);
+    if (ptr) scratch_free(ctx, ptr);
   }
   Scratch(const Scratch &) = delete;
   Scratch &operator=(const Scratch &) = delete;
@@ -236,14 +236,19 @@ inline int zero_c(phip_ctx *ctx, const Gemm &p) {
 inline int prepare_split_overwrite(phip_ctx *ctx, const Gemm &p, long tiles, size_t max_bytes, GemmArgs *a,
                                    Scratch *partials) {
   const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * a->splits;
-  if (tiles <= kTicketSlots && bytes <= max_bytes && phip_pool_alloc(ctx, bytes, &partials->ptr, nullptr) == PHIP_OK) {
-    a->atomic = 2;
-    a->partial = static_cast<float *>(partials->ptr);
-    a->tickets = ctx->tile_tickets;
-    return PHIP_OK;
+  if (ctx->fixed_mode) {
+    // an allocation-free call keeps the deterministic exchange or fails; it never changes the arithmetic
+    if (tiles > kTicketSlots) return fail(PHIP_ERR_INVALID_ARGUMENT, "%ld output tiles exceed the %d tile counters of an allocation-free call", tiles, kTicketSlots);
+    const int rc = scratch_alloc(ctx, bytes, &partials->ptr);
+    if (rc != PHIP_OK) return rc;
+  } else if (!(tiles <= kTicketSlots && bytes <= max_bytes && scratch_alloc(ctx, bytes, &partials->ptr) == PHIP_OK)) {
+    partials->ptr = nullptr;
+    return zero_c(ctx, p);
   }
-  partials->ptr = nullptr;
-  return zero_c(ctx, p);
+  a->atomic = 2;
+  a->partial = static_cast<float *>(partials->ptr);
+  a->tickets = tile_tickets(ctx);
+  return PHIP_OK;
 }
 
 }  // namespace

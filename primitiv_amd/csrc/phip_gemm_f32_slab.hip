@@ -285,7 +285,7 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   Scratch padded(ctx);
   const int kp = (p.K + 3) / 4 * 4;
   if (!vec_b && p.batch == 1 && p.rbatch == 1 && (long)p.N * kp * 4 <= (1L << 20) &&
-      phip_pool_alloc(ctx, sizeof(float) * (size_t)p.N * kp, &padded.ptr, nullptr) == PHIP_OK) {
+      scratch_alloc(ctx, sizeof(float) * (size_t)p.N * kp, &padded.ptr) == PHIP_OK) {
     const int total = p.N * kp;
     hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0,
                        ctx->stream, b_ptr, p.ldb, static_cast<float *>(padded.ptr), kp, p.N, p.K);

@@ -40,6 +40,13 @@ struct phip_ctx {
   // One counter per output tile of a launch whose workgroups share tiles (see
   // phip::kTicketSlots); all zero between launches.
   uint32_t *tile_tickets = nullptr;
+  // Allocation-free calls (phip_matmul_fw_f32_noalloc): this device's copy of the
+  // library's fixed scratch array, how much of it the running call has handed out,
+  // and whether such a call is running (scratch then comes from there, see
+  // phip::scratch_alloc).
+  unsigned char *fixed_scratch = nullptr;
+  size_t fixed_used = 0;
+  bool fixed_mode = false;
 };
 
 struct phip_event {
@@ -76,6 +83,17 @@ namespace phip {
 
 // Entries of phip_ctx::tile_tickets.
 constexpr int kTicketSlots = 65536;
+
+// Scratch memory of a launch (partial tiles of a split product, a padded copy of
+// a small operand): a pool block, or, during an allocation-free call, a piece of
+// the device's fixed scratch array (no allocation; fails with a message when the
+// call needs more than kFixedScratchBytes in total).  scratch_free returns a pool
+// block; the stream is in order, so the block may be reused behind the launches
+// that read it.  tile_tickets gives the zeroed per-tile counters that go with it.
+constexpr size_t kFixedScratchBytes = 16u << 20;
+int scratch_alloc(phip_ctx *ctx, size_t bytes, void **out);
+void scratch_free(phip_ctx *ctx, void *ptr);
+uint32_t *tile_tickets(phip_ctx *ctx);
 
 // Bits of phip_ctx::lds_limit_raised: first slot of each kernel family that
 // asks for a dynamic LDS size (one slot per instantiation, counted from here).

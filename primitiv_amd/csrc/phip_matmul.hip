@@ -172,6 +172,19 @@ int phip_matmul_fw_bf16(phip_ctx *ctx, const void *a, const void *b, void *y, ui
   return matmul_fw(ctx, Elem::BF16, a, b, y, di, dj, dk, ba, bb);
 }
 
+int phip_matmul_fw_f32_noalloc(phip_ctx *ctx, const float *a, const float *b, float *y, uint32_t di,
+                               uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  PHIP_REQUIRE(ctx->fixed_scratch != nullptr, "device %d has no fixed scratch array", ctx->device);
+  // every piece of scratch memory that the launchers ask for now comes out of the fixed array
+  struct Mode {
+    phip_ctx *ctx;
+    explicit Mode(phip_ctx *c) : ctx(c) { ctx->fixed_mode = true; ctx->fixed_used = 0; }
+    ~Mode() { ctx->fixed_mode = false; }
+  } mode(ctx);
+  return matmul_fw(ctx, Elem::F32, a, b, y, di, dj, dk, ba, bb);
+}
+
 int phip_matmul_bw_f32(phip_ctx *ctx, const float *a, const float *b, const float *gy, float *ga,
                        float *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
   return matmul_bw(ctx, Elem::F32, a, b, gy, ga, gb, di, dj, dk, ba, bb);

@@ -25,6 +25,57 @@ static std::mutex g_registry_mutex;
 static std::unordered_map<uint64_t, phip_ctx *> g_registry;
 static std::atomic<uint64_t> g_next_id{1};
 
+// Scratch of the allocation-free entry points: tile counters, then kFixedScratchBytes
+// for partial tiles and operand copies.  Every GPU holds its own copy of the array
+// at its own address until the process ends; `scratch` itself is only the host-side
+// name of the symbol, g_fixed_scratch[device] the device address.  Device arrays
+// start zeroed, and every launch leaves the counters it used zeroed again.
+constexpr size_t kFixedTicketBytes = sizeof(uint32_t) * kTicketSlots;
+static __device__ __align__(256) unsigned char scratch[kFixedTicketBytes + kFixedScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::mutex g_fixed_scratch_mutex;
+static unsigned char *g_fixed_scratch[kMaxDevices] = {};
+
+// Device address of this device's copy of `scratch`; looked up once per device, with that device current.
+static int fixed_scratch_of(int device, unsigned char **out) {
+  *out = nullptr;
+  if (device < 0 || device >= kMaxDevices) return PHIP_OK;  // no allocation-free calls on such a device
+  std::lock_guard<std::mutex> lock(g_fixed_scratch_mutex);
+  if (g_fixed_scratch[device] == nullptr) {
+    PHIP_HIP(hipSetDevice(device));
+    void *ptr = nullptr;
+    PHIP_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_fixed_scratch[device] = static_cast<unsigned char *>(ptr);
+  }
+  *out = g_fixed_scratch[device];
+  return PHIP_OK;
+}
+
+int scratch_alloc(phip_ctx *ctx, size_t bytes, void **out) {
+  if (!ctx->fixed_mode) return phip_pool_alloc(ctx, bytes, out, nullptr);
+  *out = nullptr;
+  const size_t start = (ctx->fixed_used + 255) / 256 * 256;
+  if (bytes > kFixedScratchBytes || start > kFixedScratchBytes - bytes) {
+    return fail(PHIP_ERR_INVALID_ARGUMENT,
+                "this product needs %zu bytes of scratch memory on top of %zu; an allocation-free call has %zu",
+                bytes, start, kFixedScratchBytes);
+  }
+  *out = ctx->fixed_scratch + kFixedTicketBytes + start;
+  ctx->fixed_used = start + bytes;
+  return PHIP_OK;
+}
+
+void scratch_free(phip_ctx *ctx, void *ptr) {
+  if (ptr == nullptr) return;
+  const unsigned char *p = static_cast<const unsigned char *>(ptr);
+  if (ctx->fixed_scratch && p >= ctx->fixed_scratch && p < ctx->fixed_scratch + kFixedTicketBytes + kFixedScratchBytes) return;
+  (void)phip_pool_free(ctx, ptr);
+}
+
+uint32_t *tile_tickets(phip_ctx *ctx) {
+  return ctx->fixed_mode ? reinterpret_cast<uint32_t *>(ctx->fixed_scratch) : ctx->tile_tickets;
+}
+
 static unsigned ceil_log2(uint64_t x) {
   unsigned s = 0;
   while ((1ull << s) < x) ++s;
@@ -105,6 +156,11 @@ int phip_ctx_create(int device_id, phip_ctx **out) {
   PHIP_HIP(hipSetDevice(device_id));
   phip_ctx *ctx = new phip_ctx();
   ctx->device = device_id;
+  rc = phip::fixed_scratch_of(device_id, &ctx->fixed_scratch);
+  if (rc != PHIP_OK) {
+    delete ctx;
+    return rc;
+  }
   hipError_t e = hipGetDeviceProperties(&ctx->prop, device_id);
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->tile_tickets), sizeof(uint32_t) * phip::kTicketSlots);
