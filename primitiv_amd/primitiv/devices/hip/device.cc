@@ -212,11 +212,21 @@ HIP::HIP(std::uint32_t device_id, std::uint32_t rng_seed, Storage storage)
   phip_ctx *ctx = ctx_;
   // The pool asks libphip for raw blocks; a failed allocation must throw so
   // that the pool releases its idle blocks and retries
-  // (primitiv/core/memory_pool.cc:53-63).
+  // (primitiv/core/memory_pool.cc:53-63).  libphip keeps a pool of its own
+  // for the scratch memory of its kernels (power-of-two blocks, cached when
+  // idle): when the device is full those blocks are given back first.
   pool_.reset(new MemoryPool(
       [ctx](std::size_t size) -> void * {
         void *ptr = nullptr;
-        PHIP_CALL(::phip_malloc(ctx, size, &ptr));
+        int status = ::phip_malloc(ctx, size, &ptr);
+        if (status == PHIP_ERR_OUT_OF_MEMORY) {
+          PHIP_CALL(::phip_pool_release_reserved(ctx));
+          status = ::phip_malloc(ctx, size, &ptr);
+        }
+        if (status != PHIP_OK) {
+          PRIMITIV_THROW_ERROR(
+              "libphip call failed. statement: phip_malloc, status: " << status << ": " << ::phip_last_error());
+        }
         return ptr;
       },
       [ctx](void *ptr) -> void {

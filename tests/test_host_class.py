@@ -1,6 +1,7 @@
-"""The C++ devices::HIP class must compile, warning-free, against the real
-primitiv headers.  Runs only where the reference tree and g++ are present (it
-is never available on a GPU box); nothing is linked or executed."""
+"""Every pure virtual of primitiv::Device must be overridden by the C++ classes.
+Runs only where the reference tree and g++ are present (never on a GPU box).
+The class itself is compiled with -Wall -Wextra -Werror, linked and run by
+test_host_class_runs.py."""
 import os
 import shutil
 import subprocess
@@ -9,16 +10,6 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = os.environ.get("PRIMITIV_SOURCE_DIR", "/root/reference")
-
-
-@pytest.mark.skipif(not os.path.isdir(os.path.join(REF, "primitiv", "core")) or not shutil.which("g++"),
-                    reason="needs the primitiv source tree and g++")
-def test_hip_device_class_compiles_against_primitiv_headers():
-    src = os.path.join(ROOT, "primitiv_amd", "primitiv", "devices", "hip", "device.cc")
-    cmd = ["g++", "-std=c++11", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
-           "-I" + REF, "-I" + os.path.join(ROOT, "primitiv_amd"), "-I" + os.path.join(ROOT, "include"), src]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    assert res.returncode == 0, res.stderr
 
 
 @pytest.mark.skipif(not os.path.isdir(os.path.join(REF, "primitiv", "core")) or not shutil.which("g++"),
