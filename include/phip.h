@@ -85,7 +85,9 @@ int phip_sync(phip_ctx *ctx);
  * Reference: the allocator / deleter lambdas handed to MemoryPool
  * (primitiv/internal/cuda/utils.h:330-340).  phip_malloc fails with
  * PHIP_ERR_OUT_OF_MEMORY so the caller's pool can release blocks and retry
- * (primitiv/core/memory_pool.cc:53-63). */
+ * (primitiv/core/memory_pool.cc:53-63).  Before it gives up, phip_malloc
+ * frees the idle blocks of the pooled memory below (every context on the same
+ * GPU) and tries once more. */
 int phip_malloc(phip_ctx *ctx, size_t bytes, void **out);
 int phip_free(phip_ctx *ctx, void *ptr);
 
@@ -94,7 +96,11 @@ int phip_free(phip_ctx *ctx, void *ptr);
  * (primitiv/core/memory_pool.cc:35-95): request rounded up to a power of two
  * (at least `2*sizeof(float)`, primitiv/internal/cuda/utils.h:337-342),
  * per-size free lists, one retry after releasing the reserved blocks.
- * bytes == 0 yields *out = NULL, *allocated = 0. */
+ * bytes == 0 yields *out = NULL, *allocated = 0.  The library takes the scratch
+ * memory of its own kernels from the same pool (partial tiles of split
+ * products, unfolded images, a transposed 16-bit operand), so those blocks are
+ * powers of two as well and stay cached until released; the retry releases
+ * the idle blocks of every context on the GPU. */
 int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated);
 int phip_pool_free(phip_ctx *ctx, void *ptr);
 /* Same as phip_pool_free but addressed by context id; succeeds silently when

@@ -25,6 +25,7 @@ SOURCES = [
     "phip_gemm_f32_slab.hip",
     "phip_gemm_f32_rankk.hip",
     "phip_gemm_f32_pair.hip",
+    "phip_gemm_f32_stream_pair.hip",
     "phip_conv_pool.hip",
     "phip_gemm_h16.hip",
     "phip_gemm_h16_big.hip",

@@ -181,6 +181,17 @@ __device__ inline void sum_partials(const GemmArgs &g, int z, int row0, int col0
 }
 
 // Called by all threads of the workgroup after their store_partial calls.
+// Ordering, spelled out (the exchange deliberately uses no agent-scope release /
+// acquire fences, which on this part write back and invalidate a whole L2):
+//  * the partial tiles are written and read by agent-scope atomic accesses, which
+//    bypass the per-XCD L2s, so no cache can hold a stale copy of them;
+//  * s_waitcnt vmcnt(0) holds every lane until its own such stores are acknowledged
+//    by memory, and its "memory" clobber keeps the compiler from moving them below;
+//  * __syncthreads() (a workgroup-scope release / acquire fence and a barrier) puts
+//    all lanes' acknowledged stores before thread 0's ticket, and, after the second
+//    barrier, keeps the loads of sum_partials from being moved above the ticket;
+//  * the ticket is an agent-scope atomic on one address: whoever draws the last one
+//    does so after every other workgroup's stores were acknowledged.
 __device__ inline bool last_of_tile(const GemmArgs &g, int tile_id, uint32_t *flag) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own partial results have arrived, before the ticket
   __syncthreads();

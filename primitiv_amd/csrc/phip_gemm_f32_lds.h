@@ -99,38 +99,20 @@ struct DmaLoader {
     const uint32_t o = in ? off[q] + (uint32_t)kt_in_r * step : kOutOfRange;
     lds_dma_b128(rsrc, region_addr + (uint32_t)(wave * kInstr + q) * 1024u, o);
   }
-};
 
-// A k-contiguous operand whose rows are not 16-byte aligned (leading dimension
-// or K not a multiple of 4): the same LDS image built from 4-byte loads, 256
-// bytes (2 rows) per instruction, ROWS / 8 instructions per wavefront, every
-// element range-checked on its own.
-template <int ROWS>
-struct DmaLoaderDword {
-  static constexpr int kInstr = ROWS / 8;
-  uint32_t off[kInstr];  // byte offset of this lane's element per instruction, at K tile 0
-  int kc[kInstr];        // its k inside the tile
-  uint32_t in_mask;      // bit q: the row exists
-
-  __device__ inline void init(long ld, int x0, int X, int wave, int lane) {
-    in_mask = 0;
+  // (k-contiguous, K not a multiple of four) After instruction q of K tile kt_in_r has landed in
+  // `region`: if this lane's chunk holds k = K-1, its elements from k = K on came from the next row
+  // of the operand; they become zeros, so that they meet the other operand's zeros as zeros.
+  __device__ inline void zero_tail(unsigned char *region, int wave, int q, int lane, int kt_in_r, int K) const {
+    if constexpr (KMAJOR) {
+      const int k0 = kt_in_r * LBK + kc[q];
+      if (k0 < K && K < k0 + 4) {
+        float *chunk = reinterpret_cast<float *>(region + (wave * kInstr + q) * 1024 + lane * 16);
 #pragma unroll
-    for (int q = 0; q < kInstr; ++q) {
-      const int blk = wave * kInstr + q;  // which 256-byte block of the region
-      const int x = blk * 2 + (lane >> 5);
-      const int pos = (lane & 31) >> 2;   // chunk position inside the row's image
-      const int c = pos ^ ((x >> 1) & 7);
-      kc[q] = c * 4 + (lane & 3);
-      off[q] = (uint32_t)(((long)(x0 + x) * ld + kc[q]) * 4);
-      if (x0 + x < X) in_mask |= 1u << q;
+        for (int e = 1; e < 4; ++e)
+          if (k0 + e >= K) chunk[e] = 0.0f;
+      }
     }
-  }
-
-  __device__ inline void issue(uint4v rsrc, uint32_t region_addr, int wave, int q, int kt_in_r, int K,
-                               bool live) const {
-    const bool in = live && ((in_mask >> q) & 1u) && kt_in_r * LBK + kc[q] < K;
-    const uint32_t o = in ? off[q] + (uint32_t)kt_in_r * (uint32_t)(LBK * 4) : kOutOfRange;
-    lds_dma_b32(rsrc, region_addr + (uint32_t)(wave * kInstr + q) * 256u, o);
   }
 };
 

@@ -100,8 +100,9 @@ uint32_t *tile_tickets(phip_ctx *ctx);
 enum LdsSlot {
   kSlotGemmF32Lds = 0,    // 6 instantiations
   kSlotGemmH16Big = 8,    // 6
-  kSlotGemmF32Slab = 16,  // 5
-  kSlotGemmF32RankK = 21, // 2
+  kSlotGemmF32Slab = 16,  // 3
+  kSlotGemmF32RankK = 21, // 1
+  kSlotGemmF32StreamPair = 22,  // 1
   kSlotGemmH16Mid = 23,   // 6
 };
 
@@ -156,6 +157,9 @@ int gemm_f32_rankk(phip_ctx *ctx, const Gemm &g, bool *handled);
 // for problems so small that a launch is mostly its fixed latency.  Sets
 // *handled when it launched both; otherwise nothing has been done.
 int gemm_f32_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *handled);
+// The same for a rank-K update of a large matrix beside a product that streams a large operand
+// (the gradients of an output projection): one grid, all of it resident at once.
+int gemm_f32_stream_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *handled);
 // An operand of at least this many bytes, read once against few output columns,
 // is worth the streaming kernel (gemm_f32_slab).
 constexpr long kStreamedOperandBytes = 8L << 20;

@@ -146,6 +146,8 @@ static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, con
       bool handled = false;
       rc = gemm_f32_pair(ctx, p, q, &handled);
       if (rc != PHIP_OK || handled) return rc;
+      rc = gemm_f32_stream_pair(ctx, p, q, &handled);
+      if (rc != PHIP_OK || handled) return rc;
     }
   }
   rc = gemm_dispatch(ctx, p, elem);

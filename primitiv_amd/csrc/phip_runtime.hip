@@ -95,6 +95,20 @@ static int release_reserved_locked(phip_ctx *ctx) {
   return rc;
 }
 
+// Drains and empties the free lists of every live context on `device`.  Takes the
+// registry's lock, then each context's: the caller holds neither.
+static void release_reserved_on_device(int device) {
+  std::lock_guard<std::mutex> reg(g_registry_mutex);
+  for (auto &kv : g_registry) {
+    phip_ctx *c = kv.second;
+    if (c->device != device) continue;
+    // idle blocks may still be read by kernels enqueued before they were freed
+    (void)hipStreamSynchronize(c->stream);
+    std::lock_guard<std::mutex> lock(c->mutex);
+    (void)release_reserved_locked(c);
+  }
+}
+
 static int pool_free_locked(phip_ctx *ctx, void *ptr) {
   auto it = ctx->pool.supplied.find(ptr);
   if (it == ctx->pool.supplied.end()) {
@@ -268,6 +282,12 @@ int phip_malloc(phip_ctx *ctx, size_t bytes, void **out) {
   *out = nullptr;
   if (bytes == 0) return PHIP_OK;
   hipError_t e = hipMalloc(out, bytes);
+  if (e == hipErrorOutOfMemory) {
+    // the scratch pools of this GPU's contexts may hold idle blocks (powers of two, up to GiBs)
+    (void)hipGetLastError();
+    phip::release_reserved_on_device(ctx->device);
+    e = hipMalloc(out, bytes);
+  }
   if (e != hipSuccess) {
     (void)hipGetLastError();
     *out = nullptr;
@@ -298,19 +318,22 @@ int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated) 
   }
   const unsigned shift = phip::ceil_log2(bytes);
   const size_t block = 1ull << shift;
-  std::lock_guard<std::mutex> lock(ctx->mutex);
   void *ptr = nullptr;
-  auto &list = ctx->pool.reserved[shift];
-  if (!list.empty()) {
-    ptr = list.back();
-    list.pop_back();
-  } else {
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    auto &list = ctx->pool.reserved[shift];
+    if (!list.empty()) {
+      ptr = list.back();
+      list.pop_back();
+    }
+  }
+  if (ptr == nullptr) {
     hipError_t e = hipMalloc(&ptr, block);
     if (e != hipSuccess) {
-      // Most likely out of memory: give back every idle block and try again.
+      // Most likely out of memory: give back every idle block of every context on this GPU (a fp32 and a
+      // 16-bit device object on one GPU each have a pool) and try again.
       (void)hipGetLastError();
-      (void)hipStreamSynchronize(ctx->stream);
-      phip::release_reserved_locked(ctx);
+      phip::release_reserved_on_device(ctx->device);
       e = hipMalloc(&ptr, block);
     }
     if (e != hipSuccess) {
@@ -320,7 +343,10 @@ int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated) 
                   hipGetErrorString(e));
     }
   }
-  ctx->pool.supplied.emplace(ptr, shift);
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->pool.supplied.emplace(ptr, shift);
+  }
   *out = ptr;
   if (allocated) *allocated = block;
   return PHIP_OK;

@@ -92,6 +92,31 @@ def test_allocated_size_and_pool(devs, golden):
     _lib.call("phip_pool_release_reserved", d.ctx())
 
 
+def test_out_of_memory_reclaims_idle_blocks_of_every_context_on_the_gpu(devs):
+    # a fp32 and a 16-bit device object on one GPU each cache idle blocks; when an allocation fails, the retry
+    # (primitiv/core/memory_pool.cc:53-63) must be able to use what the other one holds
+    a, b = devs[0], devs[1]
+
+    def reserved(d):
+        sup, res = ctypes.c_uint64(), ctypes.c_uint64()
+        _lib.call("phip_pool_stats", d.ctx(), ctypes.byref(sup), ctypes.byref(res))
+        return res.value
+
+    p = ctypes.c_void_p()
+    _lib.call("phip_pool_alloc", a.ctx(), 1 << 20, ctypes.byref(p), None)
+    _lib.call("phip_pool_free", a.ctx(), p)
+    assert reserved(a) >= 1 << 20
+    huge = ctypes.c_void_p()
+    assert _lib.lib().phip_pool_alloc(b.ctx(), 1 << 40, ctypes.byref(huge), None) == _lib.PHIP_ERR_OUT_OF_MEMORY
+    assert reserved(a) == 0 and reserved(b) == 0
+    _lib.call("phip_pool_alloc", a.ctx(), 1 << 20, ctypes.byref(p), None)
+    _lib.call("phip_pool_free", a.ctx(), p)
+    assert _lib.lib().phip_malloc(b.ctx(), 1 << 40, ctypes.byref(huge)) == _lib.PHIP_ERR_OUT_OF_MEMORY
+    assert reserved(a) == 0
+    x = a.new_tensor_by_constant([1000], 2.0)          # both contexts still work
+    assert float(x.to_vector()[999]) == 2.0
+
+
 def test_tensor_outlives_device():
     # test/cuda_device_test.cc:66-78: dropping a tensor after its device is fine
     d = pa.HIP(0)
