@@ -23,12 +23,14 @@ namespace {
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
+
 constexpr int LBK = 32;
 constexpr uint32_t kOutOfRange = 0x80000000u;
 
 struct LdsArgs {
   GemmArgs g;
   uint32_t a_bytes, b_bytes;  // size of one sample of each operand
+  int whole_tiles;            // streamed-operand kernel: leading workgroups that take an unsplit tile each
 };
 
 __device__ inline uint4v make_rsrc_words(const float *p, uint32_t bytes) {

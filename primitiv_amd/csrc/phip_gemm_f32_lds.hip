@@ -308,6 +308,7 @@ static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, l
   a.tickets = ctx->tile_tickets;
   d->a_bytes = (uint32_t)a_bytes;
   d->b_bytes = (uint32_t)b_bytes;
+  d->whole_tiles = 0;
 }
 
 }  // namespace

@@ -5,9 +5,10 @@
 //
 // 128 x 128 output tiles.  A workgroup fetches the old C straight into the
 // accumulators and the whole K extent of both operands into LDS (all in flight
-// together), runs the matrix instructions and stores C.  A workgroup that is
-// given several tiles of one row block keeps A in LDS and fetches the next
-// tile's old C while the matrix instructions of the current tile run.
+// together), runs the matrix instructions, adds the old values and stores C: the
+// old values have the longest way to come and are not waited for before the
+// matrix instructions are done.  A workgroup that is given several tiles of
+// one row block keeps A in LDS.
 //
 // Operands travel global -> LDS by buffer loads that write LDS directly, 16
 // bytes per lane; such a load needs no more than 4-byte alignment, so rows of
@@ -64,16 +65,16 @@ __device__ inline void fetch_c(const TileOfC &t, float4v (&raw)[16]) {
   for (int v = 0; v < 16; ++v) raw[v] = *t.at(v);
 }
 
-// The fetched values as accumulators (zeros outside the matrix).
-__device__ inline void seed_acc(const TileOfC &t, const float4v (&raw)[16], float16v (&acc)[4]) {
+// Adds the fetched values to the accumulators (elements outside the matrix are never stored).
+__device__ inline void add_old(const TileOfC &t, const float4v (&raw)[16], float16v (&acc)[4]) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    const bool ok = t.ok(v);
-    acc[0][v] = ok ? raw[v].x : 0.0f;
-    acc[1][v] = ok ? raw[v].y : 0.0f;
-    acc[2][v] = ok ? raw[v].z : 0.0f;
-    acc[3][v] = ok ? raw[v].w : 0.0f;
+    acc[0][v] += raw[v].x;
+    acc[1][v] += raw[v].y;
+    acc[2][v] += raw[v].z;
+    acc[3][v] += raw[v].w;
   }
+  (void)t;
 }
 
 __device__ inline void store_c(const TileOfC &t, const float16v (&acc)[4]) {
@@ -97,25 +98,10 @@ __device__ inline void rankk_tiles(const LdsArgs &d, unsigned char *lds, int z, 
   const int n_kt = (g.K + LBK - 1) / LBK;
   float *Cz = g.C + (long)z * g.sC;
 
-  // the old C of the first tile first: these loads have the longest way to go
-  float4v raw[16];
-  TileOfC tile = tile_of_c(Cz, g.ldc, m0, tn_first * RBN + wave * 32, lane, g.M, g.N);
-  if (g.accumulate) fetch_c(tile, raw);
-
-  DmaLoader<false, RBM> la;
-  la.init(g.lda, m0, g.M, wave, lane);
-  const uint4v rsrc_a = make_rsrc_words(g.A + (long)z * g.sA, d.a_bytes);
-#pragma unroll
-  for (int kt = 0; kt < kKTiles; ++kt) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) la.issue(rsrc_a, lds_base + (uint32_t)kt * kRegion, wave, q, kt, g.K, kt < n_kt);
-  }
-  const uint4v rsrc_b = make_rsrc_words(g.B + (long)z * g.sB, d.b_bytes);
-
-  // Fragments of k group gk (8 k) for the lane's k slots 4*(lane/32) + e: A is
-  // one 16-byte read per e (rows 4r..4r+3 = the four blocks), B one 4-byte read.
   const uint32_t a_base = (uint32_t)((4 * (lane >> 5)) * 512 + (lane & 31) * 16);
   const uint32_t b_base = (uint32_t)((4 * (lane >> 5)) * 512 + (wave * 32 + (lane & 31)) * 4);
+  // Fragments of k group gk (8 k) for the lane's k slots 4*(lane/32) + e: A is
+  // one 16-byte read per e (rows 4r..4r+3 = the four blocks), B one 4-byte read.
   auto read_a = [&](int group, int e, float4v (&fa)[4]) {
     fa[e] = *reinterpret_cast<const float4v *>(lds + (group >> 2) * kRegion + a_base + (8 * (group & 3) + e) * 512);
   };
@@ -125,8 +111,19 @@ __device__ inline void rankk_tiles(const LdsArgs &d, unsigned char *lds, int z, 
   };
   const int groups = 4 * n_kt;
 
-  for (int j = 0; j < tn_count; ++j) {
-    const int n0 = (tn_first + j) * RBN;
+  // Operands first (they come from L2 and the matrix instructions wait for nothing else), the old C
+  // behind them: its values are only needed when the tile's products are complete, and they travel
+  // while the matrix instructions run.
+  DmaLoader<false, RBM> la;
+  la.init(g.lda, m0, g.M, wave, lane);
+  const uint4v rsrc_a = make_rsrc_words(g.A + (long)z * g.sA, d.a_bytes);
+#pragma unroll
+  for (int kt = 0; kt < kKTiles; ++kt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) la.issue(rsrc_a, lds_base + (uint32_t)kt * kRegion, wave, q, kt, g.K, kt < n_kt);
+  }
+  const uint4v rsrc_b = make_rsrc_words(g.B + (long)z * g.sB, d.b_bytes);
+  auto load_b = [&](int n0) {
     DmaLoader<false, RBN> lb;
     lb.init(g.ldb, n0, g.N, wave, lane);
 #pragma unroll
@@ -135,56 +132,68 @@ __device__ inline void rankk_tiles(const LdsArgs &d, unsigned char *lds, int z, 
       for (int q = 0; q < 4; ++q)
         lb.issue(rsrc_b, lds_base + (uint32_t)(kKTiles + kt) * kRegion, wave, q, kt, g.K, kt < n_kt);
     }
-    // operands and old values of this tile are here (and the stores of the tile before have left)
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
+  };
+  load_b(tn_first * RBN);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int j = 0; j < tn_count; ++j) {
+    const int n0 = (tn_first + j) * RBN;
+    const TileOfC tile = tile_of_c(Cz, g.ldc, m0, n0 + wave * 32, lane, g.M, g.N);
+    float4v raw[16];
+    if (g.accumulate) fetch_c(tile, raw);
 
     float16v acc[4];
-    if (g.accumulate) {
-      seed_acc(tile, raw, acc);
-    } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
-    }
-    // the next tile's old values travel while this tile's matrix instructions run
-    const TileOfC cur = tile;
-    if (j + 1 < tn_count) {
-      tile = tile_of_c(Cz, g.ldc, m0, n0 + RBN + wave * 32, lane, g.M, g.N);
-      if (g.accumulate) fetch_c(tile, raw);
-    }
+      for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
 
-    // Fragments are double-buffered in registers: group g+1 is read between the
-    // matrix instructions of group g.
-    float4v fa[2][4];
-    float fb[2][4];
+    // a wavefront whose 32 columns lie outside the matrix has nothing to compute
+    if (n0 + wave * 32 < g.N) {
+      // Fragments are double-buffered in registers: group g+1 is read between the
+      // matrix instructions of group g.
+      float4v fa[2][4];
+      float fb[2][4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      read_a(0, e, fa[0]);
-      read_b(0, e, fb[0]);
-    }
-    for (int gg = 0; gg < groups; gg += 2) {
+      for (int e = 0; e < 4; ++e) {
+        read_a(0, e, fa[0]);
+        read_b(0, e, fb[0]);
+      }
+      for (int gg = 0; gg < groups; gg += 2) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int cu = h, nxt = h ^ 1;
-        // the group after this one (past the end: group 0 again, read and not used)
-        const int ng = gg + h + 1 < groups ? gg + h + 1 : 0;
+        for (int h = 0; h < 2; ++h) {
+          const int cu = h, nxt = h ^ 1;
+          // the group after this one (past the end: group 0 again, read and not used)
+          const int ng = gg + h + 1 < groups ? gg + h + 1 : 0;
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
-          const int e = q >> 2, i = q & 3;
-          // rows of the instruction's result follow n, its columns follow m
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cu][e], fa[cu][e][i], acc[i], 0, 0, 0);
-          if (q < 4) read_a(ng, q, fa[nxt]);
-          else if (q < 8) read_b(ng, q - 4, fb[nxt]);
-          __builtin_amdgcn_sched_barrier(0);
+          for (int q = 0; q < 16; ++q) {
+            const int e = q >> 2, i = q & 3;
+            // rows of the instruction's result follow n, its columns follow m
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cu][e], fa[cu][e][i], acc[i], 0, 0, 0);
+            if (q < 4) read_a(ng, q, fa[nxt]);
+            else if (q < 8) read_b(ng, q - 4, fb[nxt]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
-    store_c(cur, acc);
-    // every wave is done with B's image before the next tile's loads overwrite it
-    if (j + 1 < tn_count) __syncthreads();
+    const bool more = j + 1 < tn_count;
+    if (more) {
+      // every wave is done with B's image: the next tile's may come
+      __syncthreads();
+      load_b(n0 + RBN);
+    }
+    if (g.accumulate) add_old(tile, raw, acc);
+    if (more) {
+      // The next tile's operands have landed before this tile's stores go out: nothing then has to be
+      // waited for while stores are outstanding (loads and stores do not complete in one order).
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+    store_c(tile, acc);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // How a problem is run by this kernel.
@@ -216,6 +225,7 @@ inline bool plan_rankk(const Gemm &p, RankKPlan *plan) {
   a.tickets = nullptr;
   d.a_bytes = (uint32_t)a_bytes;
   d.b_bytes = (uint32_t)b_bytes;
+  d.whole_tiles = 0;
   plan->tiles = (long)a.tiles_m * a.tiles_n * p.batch;
   return true;
 }
