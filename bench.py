@@ -133,9 +133,10 @@ def _workload(name):
     return WORKLOADS[name]
 
 
-def measure(name, steps, warmup, skip_cpu):
+def measure(name, steps, warmup, skip_cpu, deterministic=False):
     w = _workload(name)
     dev = pa.HIP(0) if w.storage == "f32" else pa.HIP16(0, storage=w.storage)
+    dev.set_deterministic(deterministic)
     res = Resident(dev, w)
     host_s, ev_s = time_gpu(dev, res, steps, warmup)
     del res
@@ -356,6 +357,8 @@ def main():
     ap.add_argument("--workload", default="all",
                     help="all or one of: " + ", ".join(list(WORKLOADS) + ["half_storage_bf16"]))
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle")
+    ap.add_argument("--deterministic", action="store_true",
+                    help="gradients of split products added in a fixed order (phip_set_deterministic)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one streaming y += x over 64 Mi floats (reads 512 MiB, writes 256 MiB): "
                          "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
@@ -393,7 +396,7 @@ def main():
     for n in names:
         steps = args.steps if not n.startswith("half_storage") else max(1, min(args.steps, 5))
         # the CPU figure of the bf16 variant would repeat the fp16 one: same shapes, fp32 on the CPU
-        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16")
+        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16", args.deterministic)
         print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)"
               % (n, results[n]["ms_per_step"], results[n]["tflops"], 100 * results[n]["frac_mfma_peak"],
                  results[n]["gbs"], 100 * results[n]["frac_hbm_peak"]), file=sys.stderr, flush=True)

@@ -80,6 +80,17 @@ int phip_device_info_get(phip_ctx *ctx, phip_device_info *out);
  * (primitiv/devices/cuda/ops/dump_description.cu:12-40) into buf. */
 int phip_describe(phip_ctx *ctx, char *buf, size_t buf_size);
 int phip_sync(phip_ctx *ctx);
+/* Bit-reproducible gradients.  No counterpart in the reference's interface: its
+ * CPU devices add in one fixed order by construction, its CUDA device does not
+ * (atomicAdd, e.g. primitiv/devices/cuda/ops/add.cu:16-27).  By default a
+ * matmul_bw product whose contraction is cut between workgroups adds its tiles
+ * into the accumulated gradient with fp32 atomics: every run is right to
+ * rounding (about 1e-7 relative), the bits depend on the order of arrival.
+ * With on != 0 such products exchange fp32 partial tiles instead and the last
+ * workgroup of a tile adds them in a fixed order, as forward products always
+ * do: the same bits on every run, at the cost of one more round trip through
+ * memory per launch (and the two gradient products no longer share a launch). */
+int phip_set_deterministic(phip_ctx *ctx, int on);
 
 /* ---- raw memory -----------------------------------------------------------
  * Reference: the allocator / deleter lambdas handed to MemoryPool

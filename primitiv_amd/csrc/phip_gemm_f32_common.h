@@ -239,22 +239,26 @@ inline int zero_c(phip_ctx *ctx, const Gemm &p) {
   return PHIP_OK;
 }
 
-// An overwriting product whose K is split between `a->splits` workgroups per
-// tile (a->atomic == 1 on entry): fp32 partial tiles in scratch memory, summed by
-// the last workgroup of each tile (a->atomic = 2: no zero fill of C, no atomics
-// on it, one launch, the same bits on every run); without room for them, or
-// with more tiles than tickets, a zero fill of C and atomics.
-inline int prepare_split_overwrite(phip_ctx *ctx, const Gemm &p, long tiles, size_t max_bytes, GemmArgs *a,
-                                   Scratch *partials) {
+// True when a product whose K is split between workgroups has to meet through partial tiles: an
+// overwriting one always (no zero fill, no atomics on C), an accumulating one when the context asks
+// for results that are the same bits on every run.
+inline bool wants_exchange(const phip_ctx *ctx, const Gemm &p) { return !p.accumulate || ctx->deterministic; }
+
+// A product whose K is split between `a->splits` workgroups per tile (a->atomic == 1 on entry): fp32
+// partial tiles in scratch memory, summed in order by the last workgroup of each tile, which then
+// writes (or adds to) C once (a->atomic = 2: one launch, the same bits on every run).  Without room
+// for them, or with more tiles than tickets: atomics on C, behind a zero fill for an overwriting
+// product.  An allocation-free call keeps the exchange or fails.
+inline int prepare_split_exchange(phip_ctx *ctx, const Gemm &p, long tiles, size_t max_bytes, GemmArgs *a,
+                                  Scratch *partials) {
   const size_t bytes = sizeof(float) * (size_t)p.M * p.N * p.batch * a->splits;
   if (ctx->fixed_mode) {
-    // an allocation-free call keeps the deterministic exchange or fails; it never changes the arithmetic
     if (tiles > kTicketSlots) return fail(PHIP_ERR_INVALID_ARGUMENT, "%ld output tiles exceed the %d tile counters of an allocation-free call", tiles, kTicketSlots);
     const int rc = scratch_alloc(ctx, bytes, &partials->ptr);
     if (rc != PHIP_OK) return rc;
   } else if (!(tiles <= kTicketSlots && bytes <= max_bytes && scratch_alloc(ctx, bytes, &partials->ptr) == PHIP_OK)) {
     partials->ptr = nullptr;
-    return zero_c(ctx, p);
+    return p.accumulate ? PHIP_OK : zero_c(ctx, p);
   }
   a->atomic = 2;
   a->partial = static_cast<float *>(partials->ptr);

@@ -19,8 +19,8 @@ int launch_direct(phip_ctx *ctx, const Gemm &p, const DirectPlan &plan) {
   const long grid = plan.grid;
   if (grid > 0x7fffffffL) return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
   Scratch partials(ctx);
-  if (a.atomic && !p.accumulate) {
-    const int rc = prepare_split_overwrite(ctx, p, (long)a.tiles_m * a.tiles_n * p.batch, (size_t)(64L << 20), &a,
+  if (a.atomic && wants_exchange(ctx, p)) {
+    const int rc = prepare_split_exchange(ctx, p, (long)a.tiles_m * a.tiles_n * p.batch, (size_t)(64L << 20), &a,
                                            &partials);
     if (rc != PHIP_OK) return rc;
   }

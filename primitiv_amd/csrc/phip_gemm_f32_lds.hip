@@ -375,8 +375,8 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   LdsArgs d;
   fill_args(p, side, splits, total_ktiles, a_bytes, b_bytes, ctx, &d);
   Scratch partials(ctx);
-  if (splits > 1 && !p.accumulate) {
-    const int rc0 = prepare_split_overwrite(ctx, p, tiles, (size_t)(256L << 20), &d.g, &partials);
+  if (splits > 1 && wants_exchange(ctx, p)) {
+    const int rc0 = prepare_split_exchange(ctx, p, tiles, (size_t)(256L << 20), &d.g, &partials);
     if (rc0 != PHIP_OK) return rc0;
   }
 

@@ -26,8 +26,8 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   if (!plan_slab(p, ctx->prop.multiProcessorCount, 2, &plan)) return PHIP_OK;
   LdsArgs &d = plan.d;
   Scratch partials(ctx);
-  if (d.g.atomic && !p.accumulate) {
-    const int rc = prepare_split_overwrite(ctx, p, plan.tiles, (size_t)(64L << 20), &d.g, &partials);
+  if (d.g.atomic && wants_exchange(ctx, p)) {
+    const int rc = prepare_split_exchange(ctx, p, plan.tiles, (size_t)(64L << 20), &d.g, &partials);
     if (rc != PHIP_OK) return rc;
   }
 #define PHIP_SLAB_G(SLOT, AK, BKM)                                                                           \

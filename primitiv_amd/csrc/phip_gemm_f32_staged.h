@@ -335,8 +335,9 @@ inline void plan_staged(const phip_ctx *ctx, const Gemm &p, StagedPlan *plan) {
   const long t = (long)a.tiles_m * a.tiles_n * p.batch;
 
   // Split K between workgroups when the C tiles alone cannot fill the chip.
+  // (this kernel's split adds tiles with atomics: a context that wants the same bits on every run gets none)
   int splits = 1;
-  if (t < 2 * cus) {
+  if (t < 2 * cus && !ctx->deterministic) {
     const long want = (4L * cus + t - 1) / t;
     const int min_ktiles = bk >= 64 ? 2 : 4;  // K tiles per workgroup worth a launch
     long cap = a.total_ktiles / min_ktiles;

@@ -55,6 +55,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_stream_pair_kernel(const
 int gemm_f32_stream_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *handled) {
   *handled = false;
   if (!first.accumulate || !second.accumulate) return PHIP_OK;
+  // the shared launch adds the tiles of a split product with atomics
+  if (ctx->deterministic) return PHIP_OK;
   if (first.batch != 1 || second.batch != 1 || first.rbatch != 1) return PHIP_OK;
   if (!second.a_kmajor || !second.b_kmajor) return PHIP_OK;
   const int cus = ctx->prop.multiProcessorCount;

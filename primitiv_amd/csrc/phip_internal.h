@@ -44,6 +44,9 @@ struct phip_ctx {
   // library's fixed scratch array, how much of it the running call has handed out,
   // and whether such a call is running (scratch then comes from there, see
   // phip::scratch_alloc).
+  // Products whose K range is split between workgroups add their tiles to an accumulated output
+  // with fp32 atomics (any order) unless this is set (phip_set_deterministic).
+  bool deterministic = false;
   unsigned char *fixed_scratch = nullptr;
   size_t fixed_used = 0;
   bool fixed_mode = false;

@@ -268,6 +268,12 @@ int phip_describe(phip_ctx *ctx, char *buf, size_t buf_size) {
   return PHIP_OK;
 }
 
+int phip_set_deterministic(phip_ctx *ctx, int on) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  ctx->deterministic = on != 0;
+  return PHIP_OK;
+}
+
 int phip_sync(phip_ctx *ctx) {
   PHIP_ENTER(ctx);
   PHIP_HIP(hipStreamSynchronize(ctx->stream));

@@ -412,6 +412,10 @@ class HIP:
     def sync(self):
         _lib.call("phip_sync", self._ctx)
 
+    def set_deterministic(self, on=True):
+        """Gradients of split products are added in a fixed order (same bits on every run)."""
+        _lib.call("phip_set_deterministic", self._ctx, 1 if on else 0)
+
     # -- storage ----------------------------------------------------------
     def _elements_to_bytes(self, n):
         return self._ITEMSIZE * n

@@ -255,6 +255,10 @@ HIP16::HIP16(std::uint32_t device_id, std::uint32_t rng_seed)
 HIP16::HIP16(std::uint32_t device_id)
 : HIP(device_id, std::random_device()(), Storage::F16) {}
 
+void HIP::set_deterministic(bool on) {
+  PHIP_CALL(::phip_set_deterministic(ctx_, on ? 1 : 0));
+}
+
 void HIP::dump_description() const {
   char buf[2048];
   PHIP_CALL(::phip_describe(ctx_, buf, sizeof(buf)));

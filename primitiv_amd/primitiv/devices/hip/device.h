@@ -63,6 +63,12 @@ public:
   }
   Storage storage() const { return storage_; }
 
+  // Gradient products whose contraction is cut between workgroups normally add
+  // their tiles with atomics (right to rounding, bits depend on the order of
+  // arrival).  With `on` they are added in a fixed order instead: the same bits
+  // on every run, like the CPU devices, at some cost per backward call.
+  void set_deterministic(bool on);
+
 private:
   // ---- implemented -------------------------------------------------------
   std::shared_ptr<void> new_handle(const Shape &shape, std::size_t *const allocated_size) override;

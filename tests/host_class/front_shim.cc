@@ -146,6 +146,11 @@ int hc_device_dump_description(Device *dev) {
   dev->dump_description();
   HC_END
 }
+int hc_device_set_deterministic(Device *dev, int on) {
+  HC_TRY
+  static_cast<primitiv::devices::HIP *>(dev)->set_deterministic(on != 0);
+  HC_END
+}
 int hc_num_devices(U32 *out) {
   HC_TRY
   *out = primitiv::devices::HIP::num_devices();

@@ -405,6 +405,49 @@ def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
         assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), first)
 
 
+# accumulating products whose contraction is cut between workgroups: the dense layer's and the
+# recurrent gate's gradients (small, both products normally in one launch), an output projection
+# (rank-K update + streamed operand, whole and split tiles), mid-size long-K products (large tiles),
+# ragged shapes, per-sample products and a contraction over the minibatch
+SPLIT_BW = [(256, 784, 1, 1, 128), (2048, 512, 1, 1, 64), (4100, 650, 1, 1, 64), (10000, 650, 1, 1, 64),
+            (1028, 2052, 1100, 1, 1), (1536, 512, 4096, 1, 1), (96, 1000, 5, 1, 3), (48, 2048, 8, 3, 3),
+            (300, 20, 5, 9, 1), (130, 70, 258, 1, 4)]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", SPLIT_BW)
+def test_split_backward_is_reproducible(di, dj, dk, ba, bb):
+    # with phip_set_deterministic the tiles of a split product are added in a fixed order: the same bits
+    # on every run (the default adds them with atomics: right to rounding, bits vary)
+    d = pa.HIP(0)
+    d.set_deterministic(True)
+    rng = np.random.default_rng(di + dj + dk)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    ta = d.new_tensor_by_vector(pa.Shape([di, dj], ba), a)
+    tb = d.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    ty = d.matmul_fw(ta, tb)
+    tgy = d.new_tensor_by_vector(ty.shape(), gy)
+
+    def run():
+        tga = d.new_tensor_by_vector(ta.shape(), ga0)
+        tgb = d.new_tensor_by_vector(tb.shape(), gb0)
+        d.matmul_bw(ta, tb, ty, tgy, tga, tgb)
+        return tga.to_vector(), tgb.to_vector()
+
+    ga, gb = run()
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(ga, rga) <= F32_TOL and norm_rel_err(gb, rgb) <= F32_TOL
+    for _ in range(12):
+        ga2, gb2 = run()
+        assert np.array_equal(ga, ga2) and np.array_equal(gb, gb2)
+    d.close()
+
+
+
 # shapes that reach the 256x256x64 large-tile kernel with ragged edges in every
 # dimension (multiples of 8, not of 256 / 64), in each batch case
 BIG_H16 = [  # di, dj, dk, ba, bb

@@ -60,6 +60,7 @@ def test_device_identity_and_invalid_ids():
     assert d32.type() == pa.DeviceType.HIP == 0x00030000
     assert d16.type() == dbf.type() == pa.DeviceType.HIP16 == 0x00030001
     hc.call("hc_device_dump_description", d32.ptr)
+    hc.call("hc_device_set_deterministic", d32.ptr, 1)
     p = ctypes.c_void_p()
     hc.call("hc_device_new_hip16", 0, 5, ctypes.byref(p))       # the CUDA16-shaped constructor
     t = ctypes.c_uint32(0)
