@@ -31,10 +31,19 @@ from primitiv_amd.configs import WORKLOADS  # noqa: E402
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6, "bf16": 2516.6}
 PEAK_HBM_GBS = 8000.0
 HEADLINE = "square_batched"
-# HBM bytes per launch of the headline kernel (average of its three operand-layout
-# instantiations): rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors read
-# off a streaming y += x of known size (the summary under profiles/ holds both runs).
-HEADLINE_TRAFFIC_BYTES = 195.9e6 + 67.1e6
+# HBM bytes per step by rocprofv3's counters, from profiles/matmul_workloads_kernel_times_traffic_counters.txt
+# section 2: per dispatch FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (the factors read off a streaming
+# y += x of known size in the same runs), summed over a step's launches ("HBM bytes per step by the
+# counters" there).  Algorithmic bytes for comparison are Workload.bytes_per_step().
+COUNTER_TRAFFIC_BYTES_PER_STEP = {
+    "square_batched": 761.9e6,       # 206.05 + 283.50 + 272.36 MB: the three gemm_f32_lds_kernel launches
+    "dense": 11.48e6,                # gemm_f32_direct_kernel 3.95 + gemm_f32_pair_kernel 7.52 MB
+    "rnn_gate": 871.9e6,             # 30 x (9.64 + 19.43 MB)
+    "output_projection": 4474.3e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.19 MB)
+    "half_storage": 6289.5e6,        # 2 x 2122.64 + 1977.07 + 67.17 MB (transposed copy of a)
+}
+# per launch of the headline kernel (average of its three operand-layout instantiations)
+HEADLINE_TRAFFIC_BYTES = COUNTER_TRAFFIC_BYTES_PER_STEP["square_batched"] / 3
 
 
 class Resident:
@@ -93,6 +102,57 @@ def time_gpu(dev, res, steps, warmup):
     return host, ms.value * 1e-3
 
 
+class _Dims(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint32) for n in ("di", "dj", "dk", "ba", "bb")]
+
+
+_bench_lib = None
+
+
+def _native():
+    """libphip_bench.so: the same loops in native code (primitiv_amd/bench_front.cc)."""
+    global _bench_lib
+    if _bench_lib is None:
+        _lib.lib()
+        path = os.path.join(ROOT, "primitiv_amd", "libphip_bench.so")
+        if not os.path.exists(path):
+            raise _lib.Error("libphip_bench.so is not built; run `python -m primitiv_amd.build`")
+        l = ctypes.CDLL(path)
+        vp, pp, i = ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int
+        out = [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+        # device pointers are 64-bit: without these ctypes would pass them as C ints
+        l.phip_bench_raw_loop.argtypes = [vp, vp, vp, pp, pp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
+        l.phip_bench_front_loop.argtypes = [vp, vp, vp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
+        l.phip_bench_raw_loop.restype = l.phip_bench_front_loop.restype = i
+        _bench_lib = l
+    return _bench_lib
+
+
+def time_front(dev, res, steps, warmup):
+    """Per-step milliseconds of the fp32 workload `res` in native loops: the two entry points on
+    preallocated outputs ("raw", what the Python loop above times), and with what primitiv's Device
+    front does around them per call ("front": y from the pool, the per-timestep gradient from the pool
+    and zero-filled, both handed back; primitiv/core/device.cc:20-24,268-301)."""
+    w = res.w
+    n = w.steps
+    arr = lambda ptrs: (ctypes.c_void_p * n)(*ptrs)
+    b, gy = arr([p[0] for p in res.ptrs]), arr([p[1] for p in res.ptrs])
+    y, gb = arr([p[2] for p in res.ptrs]), arr([p[3] for p in res.ptrs])
+    d = _Dims(w.di, w.dj, w.dk, w.ba, w.bb)
+    ev, host = ctypes.c_float(), ctypes.c_double()
+    out = {}
+    L = _native()
+    _lib.check(L.phip_bench_raw_loop(dev.ctx(), res.a.handle(), res.ga.handle(), b, gy, y, gb, ctypes.byref(d), n,
+                                     steps, warmup, ctypes.byref(ev), ctypes.byref(host)))
+    out["ms_per_step_native_raw"] = ev.value / steps
+    out["ms_per_step_native_raw_host_clock"] = host.value / steps
+    _lib.check(L.phip_bench_front_loop(dev.ctx(), res.a.handle(), res.ga.handle(), b, gy, ctypes.byref(d), n,
+                                       steps, warmup, ctypes.byref(ev), ctypes.byref(host)))
+    out["ms_per_step_front"] = ev.value / steps
+    out["ms_per_step_front_host_clock"] = host.value / steps
+    return out
+
+
 def cpu_baseline(w, threads=1):
     """Times the CPU oracle (a port of the reference's Eigen device, one
     thread, as the reference builds Eigen without OpenMP) on a bounded sample
@@ -119,7 +179,12 @@ def cpu_baseline(w, threads=1):
             oracle.matmul_bw(a, b, gy, ga, gb, w.di, w.dj, w.dk, w.ba, bb, threads)
         best = min(best, time.perf_counter() - t0)
     flops = 3 * 2 * w.di * w.dj * w.dk * bs * steps
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count()
     return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "host_cores_online": os.cpu_count(), "host_cores_usable": usable,
             "sample": "%s, best of %d, %.2f s" % (sample, repeats, best)}
 
 
@@ -139,6 +204,7 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False):
     dev.set_deterministic(deterministic)
     res = Resident(dev, w)
     host_s, ev_s = time_gpu(dev, res, steps, warmup)
+    front = time_front(dev, res, steps, warmup) if w.storage == "f32" else {}
     del res
     dev.close()
     per_step = ev_s / steps
@@ -154,6 +220,13 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False):
         "binding_roofline": "mfma" if f_mfma >= f_hbm else "hbm",
         "frac_binding_roofline": max(f_mfma, f_hbm),
     }
+    out.update(front)
+    # HBM traffic per step by the counters (profiles/), next to the algorithmic bytes above
+    if name in COUNTER_TRAFFIC_BYTES_PER_STEP:
+        traffic = COUNTER_TRAFFIC_BYTES_PER_STEP[name]
+        out["counter_traffic_bytes_per_step"] = traffic
+        out["counter_gbs"] = traffic / per_step / 1e9
+        out["counter_frac_hbm_peak"] = traffic / per_step / 1e9 / PEAK_HBM_GBS
     if not skip_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     return out
