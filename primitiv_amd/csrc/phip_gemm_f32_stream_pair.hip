@@ -17,8 +17,6 @@
 namespace phip {
 namespace {
 
-// 64 x 64 tiles of the streamed product, five stages of A in flight (72 KiB of LDS): one such workgroup
-// per compute unit beside one of the rank-K update
 // The streamed product's workgroups as on their own: 32 x 64 tiles, four stages in flight.  64 x 64 tiles
 // with five stages of A in flight, and 32 x 64 tiles with 8 or 11, measured 1 - 3 % slower on the output
 // projection: the mix of the two products is not bound by how much of the streamed operand is in flight.

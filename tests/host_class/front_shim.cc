@@ -126,6 +126,12 @@ int hc_device_new(U32 device_id, U32 seed, U32 storage, Device **out) {
   *out = new primitiv::devices::HIP(device_id, seed, static_cast<primitiv::devices::HIP::Storage>(storage));
   HC_END
 }
+// primitiv's own plain CPU device (primitiv/devices/naive/device.h:15-28), to check the oracle against
+int hc_device_new_naive(U32 seed, Device **out) {
+  HC_TRY
+  *out = new primitiv::devices::Naive(seed);
+  HC_END
+}
 int hc_device_new_hip16(U32 device_id, U32 seed, Device **out) {
   HC_TRY
   *out = new primitiv::devices::HIP16(device_id, seed);

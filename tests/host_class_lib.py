@@ -269,7 +269,8 @@ def _shape_args(shape):
 
 
 class HostDevice:
-    """A primitiv::devices::HIP object behind the Python mirror's method names."""
+    """A primitiv::devices::HIP object (or, with storage "naive", primitiv's own CPU device) behind
+    the Python mirror's method names."""
 
     UNARY_OPS = ("negate", "abs", "sqrt", "exp", "log", "tanh", "sigmoid", "softplus", "sin", "cos", "tan")
 
@@ -277,7 +278,10 @@ class HostDevice:
         self.storage = storage
         self._SUFFIX = storage
         self.ptr = _vp()
-        if via_c_api:
+        if storage == "naive":
+            # primitiv's own CPU device behind the same wrapper
+            call("hc_device_new_naive", _u32(seed), ctypes.byref(self.ptr))
+        elif via_c_api:
             if storage == "f32":
                 c_api("primitivCreateHipDeviceWithSeed", _u32(device_id), _u32(seed), ctypes.byref(self.ptr))
             else:
