@@ -79,15 +79,30 @@ class Resident:
                 _lib.check(rc)
 
 
+# The GPU's clocks take tens of milliseconds of load to settle (square_batched: 114 TFLOP/s behind
+# 3 warm-up steps of 0.9 ms, 122 behind 10, 129.6 behind 30 or 100): the untimed warm-up is the
+# requested number of steps and at least this much time.
+WARMUP_MIN_SECONDS = 0.06
+
+
+def _warm_up(dev, step, warmup):
+    t0 = time.perf_counter()
+    for _ in range(warmup):
+        step()
+    dev.sync()
+    while time.perf_counter() - t0 < WARMUP_MIN_SECONDS:
+        for _ in range(8):
+            step()
+        dev.sync()
+
+
 def time_gpu(dev, res, steps, warmup):
     """(host seconds, event seconds) for `steps` steps."""
     ctx = dev.ctx()
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     _lib.call("phip_event_create", ctx, ctypes.byref(e0))
     _lib.call("phip_event_create", ctx, ctypes.byref(e1))
-    for _ in range(warmup):
-        res.step()
-    dev.sync()
+    _warm_up(dev, res.step, warmup)
     t0 = time.perf_counter()
     _lib.call("phip_event_record", ctx, e0)
     for _ in range(steps):
@@ -198,13 +213,21 @@ def _workload(name):
     return WORKLOADS[name]
 
 
-def measure(name, steps, warmup, skip_cpu, deterministic=False):
+def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False):
     w = _workload(name)
     dev = pa.HIP(0) if w.storage == "f32" else pa.HIP16(0, storage=w.storage)
     dev.set_deterministic(deterministic)
+    dev.set_overlap(not in_order)
     res = Resident(dev, w)
     host_s, ev_s = time_gpu(dev, res, steps, warmup)
     front = time_front(dev, res, steps, warmup) if w.storage == "f32" else {}
+    if w.storage == "f32":
+        # the same loop with every launch on one stream: what the library's second lane for runs of
+        # independent matmul calls (phip_set_overlap) contributes to ms_per_step
+        dev.set_overlap(False)
+        _, in_order_s = time_gpu(dev, res, steps, warmup)
+        dev.set_overlap(not in_order)
+        front["ms_per_step_in_order"] = in_order_s / steps * 1e3
     del res
     dev.close()
     per_step = ev_s / steps
@@ -430,6 +453,8 @@ def main():
     ap.add_argument("--workload", default="all",
                     help="all or one of: " + ", ".join(list(WORKLOADS) + ["half_storage_bf16"]))
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle")
+    ap.add_argument("--in-order", action="store_true",
+                    help="every launch on one stream (phip_set_overlap off): per-kernel durations under a profiler")
     ap.add_argument("--deterministic", action="store_true",
                     help="gradients of split products added in a fixed order (phip_set_deterministic)")
     ap.add_argument("--traffic-calibration", action="store_true",
@@ -469,10 +494,12 @@ def main():
     for n in names:
         steps = args.steps if not n.startswith("half_storage") else max(1, min(args.steps, 5))
         # the CPU figure of the bf16 variant would repeat the fp16 one: same shapes, fp32 on the CPU
-        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16", args.deterministic)
-        print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)"
+        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16", args.deterministic, args.in_order)
+        print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)%s"
               % (n, results[n]["ms_per_step"], results[n]["tflops"], 100 * results[n]["frac_mfma_peak"],
-                 results[n]["gbs"], 100 * results[n]["frac_hbm_peak"]), file=sys.stderr, flush=True)
+                 results[n]["gbs"], 100 * results[n]["frac_hbm_peak"],
+                 "  [%.3f ms/step with every launch on one stream]" % results[n]["ms_per_step_in_order"]
+                 if "ms_per_step_in_order" in results[n] else ""), file=sys.stderr, flush=True)
 
     head = results.get(HEADLINE) or results[names[0]]
     w = WORKLOADS[head["workload"]]

@@ -91,6 +91,19 @@ int phip_sync(phip_ctx *ctx);
  * do: the same bits on every run, at the cost of one more round trip through
  * memory per launch (and the two gradient products no longer share a launch). */
 int phip_set_deterministic(phip_ctx *ctx, int on);
+/* Two lanes for matrix products.  No counterpart in the reference's interface
+ * (its CUDA device enqueues everything on one stream).  A context runs matmul
+ * calls that follow one another and do not touch each other's operands on two
+ * streams at once - per-timestep products leave most of the GPU idle for most
+ * of their launch - and keeps what the caller observes in the order of its
+ * calls: a product waits for every earlier one whose operands it overlaps in
+ * memory, and every other operation (elementwise work, copies, phip_sync,
+ * phip_event_record) waits for both lanes.  Products of more than 4 GFLOP and
+ * allocation-free calls always run in order.  on == 0 puts every launch back
+ * on one stream; the environment variable PHIP_OVERLAP=0 makes that the
+ * default of contexts created afterwards.  The call itself waits for neither
+ * lane on the host. */
+int phip_set_overlap(phip_ctx *ctx, int on);
 
 /* ---- raw memory -----------------------------------------------------------
  * Reference: the allocator / deleter lambdas handed to MemoryPool

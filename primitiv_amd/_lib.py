@@ -58,6 +58,7 @@ SIGNATURES = {
     "phip_ctx_destroy": [_vp],
     "phip_ctx_id": [_vp],
     "phip_set_deterministic": [_vp, _int],
+    "phip_set_overlap": [_vp, _int],
     "phip_device_info_get": [_vp, ctypes.POINTER(DeviceInfo)],
     "phip_describe": [_vp, ctypes.c_char_p, _sz],
     "phip_sync": [_vp],

@@ -15,6 +15,7 @@ BENCH_LIB_PATH = os.path.join(HERE, "libphip_bench.so")
 
 SOURCES = [
     "phip_runtime.hip",
+    "phip_lanes.hip",
     "phip_elementwise.hip",
     "phip_pointwise_unary.hip",
     "phip_pointwise_binary.hip",

@@ -25,6 +25,30 @@ struct Pool {
   static constexpr size_t kMinimumSize = 2 * sizeof(float);
 };
 
+// Two lanes for matrix products (phip_lanes.hip).  In a long enough run of matmul calls, calls that
+// do not touch each other's operands run on two streams at once: the context's own (the main lane,
+// which also carries every other operation) and that of a second, private context (the side lane,
+// with its own scratch pool and tile counters, so that launches on the two lanes share nothing).
+// What the caller observes is the order of its calls.
+struct MemRange {
+  uintptr_t lo, hi;
+  bool write;
+};
+struct Lanes {
+  phip_ctx *side = nullptr;
+  bool enabled = true;
+  hipEvent_t main_tail = nullptr, side_tail = nullptr;
+  // operands of the products enqueued on a lane and not yet ordered before the other lane
+  std::vector<MemRange> main_ops, side_ops;
+  bool engaged = false;    // the side lane is in use
+  int streak = 0;          // matmul calls since the last operation of another kind
+  int since_engaged = 0;   // of which since the lanes were engaged
+  int engage_after = 0;    // length of the run that engages the lanes (grows when engaging did not pay)
+  int engage_after_base = 0;
+  bool back_off = true;
+  int last_lane = 0;       // lane of the latest product
+};
+
 }  // namespace phip
 
 struct phip_ctx {
@@ -50,6 +74,8 @@ struct phip_ctx {
   unsigned char *fixed_scratch = nullptr;
   size_t fixed_used = 0;
   bool fixed_mode = false;
+  // The second lane for matrix products; null in the side lane's own context.
+  phip::Lanes *lanes = nullptr;
 };
 
 struct phip_event {
@@ -74,15 +100,37 @@ struct phip_event {
     if (!(cond)) return phip::fail(PHIP_ERR_INVALID_ARGUMENT, __VA_ARGS__);   \
   } while (0)
 
-// Makes the context's device current and checks the context pointer.
-#define PHIP_ENTER(ctx)                                                       \
+// Makes the context's device current and checks the context pointer: for entry points that enqueue
+// nothing (memory pool, queries) and for the matrix products, which place themselves on a lane.
+#define PHIP_ENTER_HOST(ctx)                                                  \
   PHIP_REQUIRE((ctx) != nullptr, "null context");                             \
   PHIP_HIP(hipSetDevice((ctx)->device))
+
+// The same for every entry point that enqueues work on the context's stream or waits for it: the
+// stream first waits for the matrix products that run on the side lane.
+#define PHIP_ENTER(ctx)                                                       \
+  PHIP_ENTER_HOST(ctx);                                                       \
+  do {                                                                        \
+    if ((ctx)->lanes != nullptr) {                                            \
+      const int phip_join_rc__ = phip::lanes_join(ctx);                       \
+      if (phip_join_rc__ != PHIP_OK) return phip_join_rc__;                   \
+    }                                                                         \
+  } while (0)
 
 // Checks the status of the launch that was just enqueued.
 #define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
 
 namespace phip {
+
+// phip_lanes.hip.  lanes_join: the main lane waits for everything on the side lane (no-op when
+// nothing is in flight there).  lanes_place: picks the lane of a matrix product with the given
+// operand ranges, enqueues the waits it needs and returns the context to launch it on.
+// A context with (what phip_ctx_create gives) or without a side lane of its own (phip_runtime.hip).
+int ctx_create(int device_id, bool with_lanes, phip_ctx **out);
+int lanes_create(phip_ctx *ctx);
+int lanes_destroy(phip_ctx *ctx);
+int lanes_join(phip_ctx *ctx);
+int lanes_place(phip_ctx *ctx, const MemRange *ranges, int n, bool may_overlap, phip_ctx **run_on);
 
 // Entries of phip_ctx::tile_tickets.
 constexpr int kTicketSlots = 65536;

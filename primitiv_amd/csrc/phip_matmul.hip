@@ -34,11 +34,36 @@ static int gemm_dispatch(phip_ctx *ctx, const Gemm &g, Elem elem) {
   return elem == Elem::F32 ? gemm_f32(ctx, g) : gemm_h16(ctx, g, elem);
 }
 
+// Products of up to this many floating-point operations may run beside another product on the
+// context's second lane (phip_lanes.hip); a larger one occupies every compute unit for several
+// rounds of workgroups and gains nothing from company.
+constexpr double kMaxOverlapFlop = 4e9;
+
+static MemRange range_of(const void *p, uint64_t elements, Elem elem, bool write) {
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+  return MemRange{lo, lo + (uintptr_t)(elements * (elem == Elem::F32 ? 4 : 2)), write};
+}
+
+// The context (lane) this call's launches go to.
+static int place(phip_ctx *ctx, Elem elem, const MemRange *ranges, int n, uint32_t di, uint32_t dj, uint32_t dk,
+                 uint32_t ba, uint32_t bb, phip_ctx **run_on) {
+  const double flop = 2.0 * di * dj * dk * (ba > bb ? ba : bb);
+  const bool may_overlap = elem == Elem::F32 && !ctx->fixed_mode && flop <= kMaxOverlapFlop;
+  return lanes_place(ctx, ranges, n, may_overlap, run_on);
+}
+
 static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, void *y, uint32_t di,
                      uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   int rc = check_matmul_args(a, b, y, di, dj, dk, ba, bb);
   if (rc != PHIP_OK) return rc;
+  {
+    const uint64_t bs = ba > bb ? ba : bb;
+    const MemRange ranges[3] = {range_of(a, (uint64_t)di * dj * ba, elem, false), range_of(b, (uint64_t)dj * dk * bb, elem, false),
+                                range_of(y, (uint64_t)di * dk * bs, elem, true)};
+    rc = place(ctx, elem, ranges, 3, di, dj, dk, ba, bb, &ctx);
+    if (rc != PHIP_OK) return rc;
+  }
   Gemm g;
   g.A = a; g.B = b; g.C = y;
   g.lda = di; g.ldb = dj; g.ldc = di;
@@ -86,10 +111,18 @@ static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, voi
 
 static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, const void *gy, void *ga,
                      void *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   int rc = check_matmul_args(a, b, gy, di, dj, dk, ba, bb);
   if (rc != PHIP_OK) return rc;
   PHIP_REQUIRE(ga != nullptr && gb != nullptr, "null gradient pointer");
+  {
+    const uint64_t bs = ba > bb ? ba : bb;
+    const MemRange ranges[5] = {range_of(a, (uint64_t)di * dj * ba, elem, false), range_of(b, (uint64_t)dj * dk * bb, elem, false),
+                                range_of(gy, (uint64_t)di * dk * bs, elem, false), range_of(ga, (uint64_t)di * dj * ba, elem, true),
+                                range_of(gb, (uint64_t)dj * dk * bb, elem, true)};
+    rc = place(ctx, elem, ranges, 5, di, dj, dk, ba, bb, &ctx);
+    if (rc != PHIP_OK) return rc;
+  }
 
   // ga[di x dj] += gy[di x dk] . b^T : A = gy (m-contiguous), B = b^T with
   // element (k, n) at n + k*dj (n-contiguous).

@@ -119,6 +119,45 @@ static int pool_free_locked(phip_ctx *ctx, void *ptr) {
   return PHIP_OK;
 }
 
+int ctx_create(int device_id, bool with_lanes, phip_ctx **out) {
+  PHIP_REQUIRE(out != nullptr, "null output pointer");
+  *out = nullptr;
+  int rc = phip_check_support(device_id);
+  if (rc != PHIP_OK) return rc;
+  PHIP_HIP(hipSetDevice(device_id));
+  phip_ctx *ctx = new phip_ctx();
+  ctx->device = device_id;
+  rc = phip::fixed_scratch_of(device_id, &ctx->fixed_scratch);
+  if (rc != PHIP_OK) {
+    delete ctx;
+    return rc;
+  }
+  hipError_t e = hipGetDeviceProperties(&ctx->prop, device_id);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->tile_tickets), sizeof(uint32_t) * phip::kTicketSlots);
+  if (e == hipSuccess) e = hipMemset(ctx->tile_tickets, 0, sizeof(uint32_t) * phip::kTicketSlots);
+  if (e != hipSuccess) {
+    if (ctx->tile_tickets) (void)hipFree(ctx->tile_tickets);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return fail(PHIP_ERR_RUNTIME, "context creation failed: %s", hipGetErrorString(e));
+  }
+  ctx->id = phip::g_next_id.fetch_add(1);
+  {
+    std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
+    phip::g_registry.emplace(ctx->id, ctx);
+  }
+  if (with_lanes) {
+    rc = phip::lanes_create(ctx);
+    if (rc != PHIP_OK) {
+      (void)phip_ctx_destroy(ctx);
+      return rc;
+    }
+  }
+  *out = ctx;
+  return PHIP_OK;
+}
+
 }  // namespace phip
 
 using phip::fail;
@@ -162,45 +201,16 @@ int phip_check_support(int device_id) {
   return PHIP_OK;
 }
 
-int phip_ctx_create(int device_id, phip_ctx **out) {
-  PHIP_REQUIRE(out != nullptr, "null output pointer");
-  *out = nullptr;
-  int rc = phip_check_support(device_id);
-  if (rc != PHIP_OK) return rc;
-  PHIP_HIP(hipSetDevice(device_id));
-  phip_ctx *ctx = new phip_ctx();
-  ctx->device = device_id;
-  rc = phip::fixed_scratch_of(device_id, &ctx->fixed_scratch);
-  if (rc != PHIP_OK) {
-    delete ctx;
-    return rc;
-  }
-  hipError_t e = hipGetDeviceProperties(&ctx->prop, device_id);
-  if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->tile_tickets), sizeof(uint32_t) * phip::kTicketSlots);
-  if (e == hipSuccess) e = hipMemset(ctx->tile_tickets, 0, sizeof(uint32_t) * phip::kTicketSlots);
-  if (e != hipSuccess) {
-    if (ctx->tile_tickets) (void)hipFree(ctx->tile_tickets);
-    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
-    delete ctx;
-    return fail(PHIP_ERR_RUNTIME, "context creation failed: %s", hipGetErrorString(e));
-  }
-  ctx->id = phip::g_next_id.fetch_add(1);
-  {
-    std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
-    phip::g_registry.emplace(ctx->id, ctx);
-  }
-  *out = ctx;
-  return PHIP_OK;
-}
+int phip_ctx_create(int device_id, phip_ctx **out) { return phip::ctx_create(device_id, true, out); }
 
 int phip_ctx_destroy(phip_ctx *ctx) {
   PHIP_REQUIRE(ctx != nullptr, "null context");
+  const int lanes_rc = phip::lanes_destroy(ctx);  // waits for the side lane
   {
     std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
     phip::g_registry.erase(ctx->id);
   }
-  int rc = PHIP_OK;
+  int rc = lanes_rc;
   if (hipSetDevice(ctx->device) != hipSuccess ||
       hipStreamSynchronize(ctx->stream) != hipSuccess) {
     rc = fail(PHIP_ERR_RUNTIME, "synchronisation failed while destroying the context");
@@ -283,7 +293,7 @@ int phip_sync(phip_ctx *ctx) {
 // ---- raw memory ---------------------------------------------------------------
 
 int phip_malloc(phip_ctx *ctx, size_t bytes, void **out) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   PHIP_REQUIRE(out != nullptr, "null output pointer");
   *out = nullptr;
   if (bytes == 0) return PHIP_OK;
@@ -304,7 +314,7 @@ int phip_malloc(phip_ctx *ctx, size_t bytes, void **out) {
 }
 
 int phip_free(phip_ctx *ctx, void *ptr) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   if (ptr == nullptr) return PHIP_OK;
   PHIP_HIP(hipFree(ptr));
   return PHIP_OK;
@@ -313,7 +323,7 @@ int phip_free(phip_ctx *ctx, void *ptr) {
 // ---- pool ---------------------------------------------------------------------
 
 int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   PHIP_REQUIRE(out != nullptr, "null output pointer");
   *out = nullptr;
   if (allocated) *allocated = 0;
@@ -378,6 +388,10 @@ int phip_pool_release_reserved(phip_ctx *ctx) {
   PHIP_ENTER(ctx);
   // Idle blocks may still be read by kernels enqueued before they were freed.
   PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  if (ctx->lanes != nullptr) {
+    const int rc = phip_pool_release_reserved(ctx->lanes->side);  // the side lane's scratch blocks
+    if (rc != PHIP_OK) return rc;
+  }
   std::lock_guard<std::mutex> lock(ctx->mutex);
   return phip::release_reserved_locked(ctx);
 }
@@ -426,7 +440,7 @@ int phip_memcpy_d2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
 // ---- events -------------------------------------------------------------------
 
 int phip_event_create(phip_ctx *ctx, phip_event **out) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   PHIP_REQUIRE(out != nullptr, "null output pointer");
   phip_event *ev = new phip_event();
   ev->device = ctx->device;

@@ -416,6 +416,11 @@ class HIP:
         """Gradients of split products are added in a fixed order (same bits on every run)."""
         _lib.call("phip_set_deterministic", self._ctx, 1 if on else 0)
 
+    def set_overlap(self, on=True):
+        """Matmul calls that do not touch each other's operands may run on two streams at once (the
+        default); off: every launch on one stream."""
+        _lib.call("phip_set_overlap", self._ctx, 1 if on else 0)
+
     # -- storage ----------------------------------------------------------
     def _elements_to_bytes(self, n):
         return self._ITEMSIZE * n

@@ -51,6 +51,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_rankk.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_pair.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_stream_pair.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_lanes.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_conv_pool.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16_big.hip

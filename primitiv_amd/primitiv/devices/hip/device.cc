@@ -259,6 +259,10 @@ void HIP::set_deterministic(bool on) {
   PHIP_CALL(::phip_set_deterministic(ctx_, on ? 1 : 0));
 }
 
+void HIP::set_overlap(bool on) {
+  PHIP_CALL(::phip_set_overlap(ctx_, on ? 1 : 0));
+}
+
 void HIP::dump_description() const {
   char buf[2048];
   PHIP_CALL(::phip_describe(ctx_, buf, sizeof(buf)));

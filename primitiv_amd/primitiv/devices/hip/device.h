@@ -69,6 +69,11 @@ public:
   // on every run, like the CPU devices, at some cost per backward call.
   void set_deterministic(bool on);
 
+  // Matmul calls that follow one another and do not touch each other's
+  // operands run on two streams at once (the default); what the caller observes
+  // stays in the order of its calls.  Off: every launch on one stream.
+  void set_overlap(bool on);
+
 private:
   // ---- implemented -------------------------------------------------------
   std::shared_ptr<void> new_handle(const Shape &shape, std::size_t *const allocated_size) override;

@@ -157,6 +157,11 @@ int hc_device_set_deterministic(Device *dev, int on) {
   static_cast<primitiv::devices::HIP *>(dev)->set_deterministic(on != 0);
   HC_END
 }
+int hc_device_set_overlap(Device *dev, int on) {
+  HC_TRY
+  static_cast<primitiv::devices::HIP *>(dev)->set_overlap(on != 0);
+  HC_END
+}
 int hc_num_devices(U32 *out) {
   HC_TRY
   *out = primitiv::devices::HIP::num_devices();

@@ -61,6 +61,8 @@ def test_device_identity_and_invalid_ids():
     assert d16.type() == dbf.type() == pa.DeviceType.HIP16 == 0x00030001
     hc.call("hc_device_dump_description", d32.ptr)
     hc.call("hc_device_set_deterministic", d32.ptr, 1)
+    hc.call("hc_device_set_overlap", d32.ptr, 0)
+    hc.call("hc_device_set_overlap", d32.ptr, 1)
     p = ctypes.c_void_p()
     hc.call("hc_device_new_hip16", 0, 5, ctypes.byref(p))       # the CUDA16-shaped constructor
     t = ctypes.c_uint32(0)
