@@ -117,6 +117,18 @@ struct phip_event {
     }                                                                         \
   } while (0)
 
+// For entry points that end with the host waiting for the context's stream (phip_sync, copies from
+// and to host memory): the host waits for the side lane as well, which costs no wait of one stream
+// for the other and leaves the lanes as they are.
+#define PHIP_ENTER_BLOCKING(ctx)                                              \
+  PHIP_ENTER_HOST(ctx);                                                       \
+  do {                                                                        \
+    if ((ctx)->lanes != nullptr) {                                            \
+      const int phip_join_rc__ = phip::lanes_wait_host(ctx);                  \
+      if (phip_join_rc__ != PHIP_OK) return phip_join_rc__;                   \
+    }                                                                         \
+  } while (0)
+
 // Checks the status of the launch that was just enqueued.
 #define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
 
@@ -130,6 +142,10 @@ int ctx_create(int device_id, bool with_lanes, phip_ctx **out);
 int lanes_create(phip_ctx *ctx);
 int lanes_destroy(phip_ctx *ctx);
 int lanes_join(phip_ctx *ctx);
+// The host waits for the products in flight on both lanes; the lanes stay engaged.
+int lanes_wait_host(phip_ctx *ctx);
+// What is enqueued on the main lane next comes after the side lane's work, and touches no tensor (an event).
+int lanes_order_main_after_side(phip_ctx *ctx);
 int lanes_place(phip_ctx *ctx, const MemRange *ranges, int n, bool may_overlap, phip_ctx **run_on);
 
 // Entries of phip_ctx::tile_tickets.

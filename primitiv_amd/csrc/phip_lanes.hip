@@ -16,7 +16,10 @@
 //    lanes_join).
 //  * The side lane is engaged by the kEngageAfter-th matmul call in a row (one wait: the side lane
 //    starts behind what the main lane holds so far) and released by the first operation of another
-//    kind (one wait: the main lane continues behind the side lane).  If that happens before
+//    kind that enqueues work (one wait: the main lane continues behind the side lane).  Calls that
+//    make the host wait (phip_sync, copies from and to host memory) wait for both lanes on the host
+//    and leave them engaged; phip_event_record orders the main lane behind the side lane and
+//    leaves them engaged.  If that happens before
 //    kWorthwhile products ran on the engaged lanes, the next run has to be twice as long to engage
 //    them (up to kEngageAfterMax): a caller that never issues long runs pays for one attempt.
 //  * While engaged, a product goes to the lane that holds the earlier products it overlaps in
@@ -134,6 +137,26 @@ int lanes_join(phip_ctx *ctx) {
   } else {
     l->engage_after = l->engage_after_base;
   }
+  return PHIP_OK;
+}
+
+int lanes_wait_host(phip_ctx *ctx) {
+  Lanes *l = ctx->lanes;
+  if (!l->engaged) return PHIP_OK;
+  if (!l->side_ops.empty()) PHIP_HIP(hipStreamSynchronize(l->side->stream));
+  if (!l->main_ops.empty()) PHIP_HIP(hipStreamSynchronize(ctx->stream));
+  // nothing that the lists name is in flight any more
+  l->side_ops.clear();
+  l->main_ops.clear();
+  return PHIP_OK;
+}
+
+int lanes_order_main_after_side(phip_ctx *ctx) {
+  Lanes *l = ctx->lanes;
+  if (!l->engaged || l->side_ops.empty()) return PHIP_OK;
+  const int rc = order_after(ctx->stream, l->side->stream, l->side_tail);
+  if (rc != PHIP_OK) return rc;
+  l->side_ops.clear();
   return PHIP_OK;
 }
 

@@ -285,7 +285,7 @@ int phip_set_deterministic(phip_ctx *ctx, int on) {
 }
 
 int phip_sync(phip_ctx *ctx) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_BLOCKING(ctx);
   PHIP_HIP(hipStreamSynchronize(ctx->stream));
   return PHIP_OK;
 }
@@ -412,7 +412,7 @@ int phip_pool_stats(phip_ctx *ctx, uint64_t *supplied_bytes, uint64_t *reserved_
 // ---- copies -------------------------------------------------------------------
 
 int phip_memcpy_h2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_BLOCKING(ctx);
   if (bytes == 0) return PHIP_OK;
   PHIP_REQUIRE(dst != nullptr && src != nullptr, "null pointer in h2d copy");
   PHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
@@ -421,7 +421,7 @@ int phip_memcpy_h2d(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
 }
 
 int phip_memcpy_d2h(phip_ctx *ctx, void *dst, const void *src, size_t bytes) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_BLOCKING(ctx);
   if (bytes == 0) return PHIP_OK;
   PHIP_REQUIRE(dst != nullptr && src != nullptr, "null pointer in d2h copy");
   PHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -462,8 +462,12 @@ int phip_event_destroy(phip_event *ev) {
 }
 
 int phip_event_record(phip_ctx *ctx, phip_event *ev) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   PHIP_REQUIRE(ev != nullptr, "null event");
+  if (ctx->lanes != nullptr) {
+    const int rc = phip::lanes_order_main_after_side(ctx);
+    if (rc != PHIP_OK) return rc;
+  }
   PHIP_HIP(hipEventRecord(ev->ev, ctx->stream));
   return PHIP_OK;
 }

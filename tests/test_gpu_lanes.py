@@ -243,6 +243,10 @@ def test_default_policy_long_runs_of_calls_and_runs_cut_short():
                 y = d.matmul_fw(ta, tb[i % 4])
                 d.matmul_bw(ta, tb[i % 4], y, y, ga, gb[i % 4])
                 ys.append(y)
+                if i % 5 == 4:
+                    outs.append(y.to_vector())            # a read-back in the middle of a run: the lanes stay engaged
+                if i % 11 == 10:
+                    d.sync()
             h = d.unary_fw("tanh", ys[-1])
             outs += [h.to_vector(), ys[0].to_vector()]
         return outs + [ga.to_vector()] + [g.to_vector() for g in gb]
