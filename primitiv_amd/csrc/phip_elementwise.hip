@@ -57,9 +57,22 @@ __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const T *__restric
 
 template <typename T>
 static int fill_impl(phip_ctx *ctx, void *p, float value, size_t n) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_HOST(ctx);
   if (n == 0) return PHIP_OK;
   PHIP_REQUIRE(p != nullptr, "null pointer");
+  // A fill is the one operation that sits between the matrix products of a backward pass (every
+  // gradient is reset before products are added into it) and it names its memory as they do: it
+  // takes a lane like a product instead of releasing the lanes (phip_lanes.hip).
+  // (fp32 only: the products of 16-bit storage never leave the main lane.)
+  if (sizeof(T) == sizeof(float)) {
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+    const phip::MemRange written = {lo, lo + n * sizeof(T), true};
+    const int rc = phip::lanes_place(ctx, &written, 1, n * sizeof(T) <= ((size_t)64 << 20), &ctx);
+    if (rc != PHIP_OK) return rc;
+  } else if (ctx->lanes != nullptr) {
+    const int rc = phip::lanes_join(ctx);
+    if (rc != PHIP_OK) return rc;
+  }
   hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(n, 4, ctx)), dim3(kBlock), 0, ctx->stream,
                      static_cast<T *>(p), value, n);
   PHIP_LAUNCH_CHECK();

@@ -261,3 +261,47 @@ def test_default_policy_long_runs_of_calls_and_runs_cut_short():
         finally:
             d.close()
     _same_bits(*results)
+
+
+def test_gradients_reset_between_calls_as_a_backward_pass_does():
+    # new gradient tensor, zero fill, products added into it, the tensor handed back: per timestep, as
+    # primitiv's backward pass does; the fill takes a lane like a product
+    m, k, n = 650, 650, 64
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal(m * k).astype(np.float32) / np.sqrt(k)
+    steps = 24
+    bs = [rng.standard_normal(k * n).astype(np.float32) for _ in range(4)]
+    gys = [rng.standard_normal(m * n).astype(np.float32) for _ in range(4)]
+
+    def program(d):
+        ta = d.new_tensor_by_vector(S([m, k]), a)
+        tb = [d.new_tensor_by_vector(S([k, n]), b) for b in bs]
+        tgy = [d.new_tensor_by_vector(S([m, n]), g) for g in gys]
+        ga = d.new_tensor_by_constant(S([m, k]), 0)
+        outs = []
+        for t in range(steps):
+            y = d.matmul_fw(ta, tb[t % 4])
+            gb = d.new_tensor_by_constant(S([k, n]), 0)       # pool block of the previous timestep, refilled
+            d.matmul_bw(ta, tb[t % 4], y, tgy[t % 4], ga, gb)
+            if t % 6 == 5:
+                outs += [gb.to_vector(), y.to_vector()]
+            del gb, y
+        return outs + [ga.to_vector()]
+
+    for deterministic in (True, False):
+        results = []
+        for overlap in (True, False):
+            d = pa.HIP(0)
+            d.set_deterministic(deterministic)
+            d.set_overlap(overlap)
+            try:
+                results.append([np.asarray(v, dtype=np.float32) for v in program(d)])
+            finally:
+                d.close()
+        if deterministic:
+            _same_bits(*results)
+        else:
+            for got, want in zip(*results):
+                assert norm_rel_err(got, want) <= 1e-5
+    _, gb = oracle.matmul_bw(a, bs[1], gys[1], np.zeros(m * k, np.float32), np.zeros(k * n, np.float32), m, k, n, 1, 1)
+    assert norm_rel_err(results[1][0], gb) <= 1e-4      # timestep 5 uses operands 5 % 4 = 1
