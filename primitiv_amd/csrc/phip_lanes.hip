@@ -104,6 +104,9 @@ int lanes_create(phip_ctx *ctx) {
     delete l;
     return rc;
   }
+  // the lists never grow past this: no allocation once the context exists
+  l->main_ops.reserve(kMaxTrackedRanges + 8);
+  l->side_ops.reserve(kMaxTrackedRanges + 8);
   ctx->lanes = l;
   return PHIP_OK;
 }
