@@ -98,7 +98,11 @@ int phip_set_deterministic(phip_ctx *ctx, int on);
  * of their launch - and keeps what the caller observes in the order of its
  * calls: a product waits for every earlier one whose operands it overlaps in
  * memory, and every other operation (elementwise work, copies, phip_sync,
- * phip_event_record) waits for both lanes.  Products of more than 4 GFLOP and
+ * phip_event_record) waits for both lanes.  The second stream comes into use
+ * with the sixth such call in a row and goes out of use with the first
+ * operation of another kind that enqueues work; phip_fill_f32 counts as a
+ * matmul call here (a backward pass resets every gradient before it adds
+ * products into it).  Products of more than 4 GFLOP, 16-bit storage and
  * allocation-free calls always run in order.  on == 0 puts every launch back
  * on one stream; the environment variable PHIP_OVERLAP=0 makes that the
  * default of contexts created afterwards.  The call itself waits for neither
