@@ -92,3 +92,136 @@ def test_inplace_add_and_batch_sum_match_the_reference_device(naive):
         x = _operands(rng, volume * bs, False)
         ref = naive.batch_sum_fw(naive.new_tensor_by_vector(S([volume], bs), x)).to_vector()
         assert norm_rel_err(oracle.batch_sum(x, volume, bs), ref) <= 1e-6, (volume, bs)
+
+
+# ---- the widened rows: the same call on primitiv's Naive device and on devices::HIP over the host
+# stand-in, whose arithmetic is the oracle's (tests/host_class/phip_host_stub.cc) -----------------
+
+@pytest.fixture(scope="module")
+def mine():
+    d = hc.HostDevice("f32")
+    yield d
+    d.close()
+
+
+def _ulps(a, b):
+    a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+    ia, ib = a.view(np.int32).astype(np.int64), b.view(np.int32).astype(np.int64)
+    ia = np.where(ia < 0, -(ia & 0x7fffffff), ia)
+    ib = np.where(ib < 0, -(ib & 0x7fffffff), ib)
+    d = np.abs(ia - ib)
+    d[np.isnan(a) & np.isnan(b)] = 0
+    return int(d.max()) if d.size else 0
+
+
+def _both(naive, mine, fn):
+    return np.asarray(fn(naive)), np.asarray(fn(mine))
+
+
+def test_elementwise_families_match_the_reference_device(naive, mine):
+    rng = np.random.default_rng(21)
+    shape = S([5, 3], 4)
+    x = (rng.standard_normal(60) * 1.5).astype(np.float32)
+    xp = np.abs(x) + 0.25                                   # sqrt, log, pow want positive arguments
+    gy = rng.standard_normal(60).astype(np.float32)
+    x2 = rng.standard_normal(60).astype(np.float32)
+    for op in pa.HIP.UNARY_OPS:
+        arg = xp if op in ("sqrt", "log") else x
+        def fw(d):
+            return d.unary_fw(op, d.new_tensor_by_vector(shape, arg)).to_vector()
+        def bw(d):
+            tx = d.new_tensor_by_vector(shape, arg)
+            ty = d.unary_fw(op, tx)
+            gx = d.new_tensor_by_vector(shape, gy * 0.5)   # gradients accumulate
+            d.unary_bw(op, tx, ty, d.new_tensor_by_vector(shape, gy), gx)
+            return gx.to_vector()
+        assert _ulps(*_both(naive, mine, fw)) <= 4, op      # test/test_utils.h:26-45 grants 4 on a 32-bit device
+        if op != "negate":                                  # the Device interface has no negate_bw
+            assert _ulps(*_both(naive, mine, bw)) <= 4, op
+    for op in pa.HIP.CONST_OPS:
+        arg = xp if op in ("pow_const_r", "pow_const_l") else x
+        for k in (0.75, 2.5):
+            def fw(d):
+                return d.const_fw(op, d.new_tensor_by_vector(shape, arg), k).to_vector()
+            def bw(d):
+                tx = d.new_tensor_by_vector(shape, arg)
+                ty = d.const_fw(op, tx, k)
+                gx = d.new_tensor_by_vector(shape, gy * 0.5)
+                d.const_bw(op, tx, ty, d.new_tensor_by_vector(shape, gy), k, gx)
+                return gx.to_vector()
+            assert _ulps(*_both(naive, mine, fw)) <= 4, (op, k)
+            assert _ulps(*_both(naive, mine, bw)) <= 4, (op, k)
+    for op in pa.HIP.BINARY_OPS:
+        for ba, bb in ((4, 4), (1, 4), (4, 1)):
+            a = xp[:15 * ba] if op == "pow" else x[:15 * ba]
+            b = x2[:15 * bb] + (3.0 if op == "divide" else 0.0)
+            def fw(d):
+                return d.binary_fw(op, d.new_tensor_by_vector(S([5, 3], ba), a), d.new_tensor_by_vector(S([5, 3], bb), b)).to_vector()
+            def bw(d):
+                ta, tb = d.new_tensor_by_vector(S([5, 3], ba), a), d.new_tensor_by_vector(S([5, 3], bb), b)
+                ty = d.binary_fw(op, ta, tb)
+                ga, gb = d.new_tensor_by_constant(S([5, 3], ba), 0.5), d.new_tensor_by_constant(S([5, 3], bb), -0.25)
+                d.binary_bw(op, ta, tb, ty, d.new_tensor_by_vector(S([5, 3], max(ba, bb)), gy[:15 * max(ba, bb)]), ga, gb)
+                return np.concatenate([ga.to_vector(), gb.to_vector()])
+            assert _ulps(*_both(naive, mine, fw)) <= 4, (op, ba, bb)
+            r, m = _both(naive, mine, bw)
+            assert norm_rel_err(m, r) <= 2e-6, (op, ba, bb)   # sums over the minibatch: order of addition
+
+
+def test_moving_and_reducing_operations_match_the_reference_device(naive, mine):
+    rng = np.random.default_rng(22)
+    shape = S([4, 3, 5], 2)
+    x = rng.standard_normal(120).astype(np.float32)
+    def run(fn):
+        r, m = _both(naive, mine, fn)
+        return r, m
+    for dim in (0, 1, 2):
+        for op in ("sum", "logsumexp", "max", "min"):
+            r, m = run(lambda d: d.reduce_fw(op, d.new_tensor_by_vector(shape, x), dim).to_vector())
+            if op == "logsumexp":      # log of a sum near 1 cancels to near 0: ULPs of the result mean nothing
+                assert np.max(np.abs(r - m)) <= 2e-7 * max(1.0, np.max(np.abs(r))), (op, dim)
+            else:
+                assert _ulps(r, m) <= 4, (op, dim)
+        r, m = run(lambda d: d.flip_fw(d.new_tensor_by_vector(shape, x), dim).to_vector())
+        assert np.array_equal(r, m)
+        r, m = run(lambda d: d.slice_fw(d.new_tensor_by_vector(shape, x), dim, 1, 3).to_vector())
+        assert np.array_equal(r, m)
+        r, m = run(lambda d: d.pick_fw(d.new_tensor_by_vector(shape, x), [2, 0], dim).to_vector())
+        assert np.array_equal(r, m)
+        r, m = run(lambda d: d.concat_fw([d.new_tensor_by_vector(shape, x), d.new_tensor_by_vector(shape, -x)], dim).to_vector())
+        assert np.array_equal(r, m)
+        r, m = run(lambda d: np.asarray(d.arg_extremum("max", d.new_tensor_by_vector(shape, x), dim), dtype=np.float32))
+        assert np.array_equal(r, m)
+    r, m = run(lambda d: d.permute_dims_fw(d.new_tensor_by_vector(shape, x), [2, 0, 1]).to_vector())
+    assert np.array_equal(r, m)
+    r, m = run(lambda d: d.transpose_fw(d.new_tensor_by_vector(S([4, 5], 3), x[:60])).to_vector())
+    assert np.array_equal(r, m)
+    r, m = run(lambda d: d.broadcast_fw(d.new_tensor_by_vector(S([4, 1, 5], 2), x[:40]), 1, 3).to_vector())
+    assert np.array_equal(r, m)
+    r, m = run(lambda d: d.batch_pick_fw(d.new_tensor_by_vector(S([4, 3], 5), x[:60]), [4, 0, 0]).to_vector())
+    assert np.array_equal(r, m)
+
+
+def test_convolution_and_pooling_match_the_reference_device(naive, mine):
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal(7 * 6 * 3 * 2).astype(np.float32)
+    w = rng.standard_normal(3 * 2 * 3 * 4).astype(np.float32)
+    for p in ((0, 0, 1, 1, 1, 1), (1, 1, 2, 1, 1, 1), (2, 1, 1, 2, 2, 1)):      # padding, stride, dilation
+        def fw(d):
+            return d.conv2d_fw(d.new_tensor_by_vector(S([7, 6, 3], 2), x), d.new_tensor_by_vector(S([3, 2, 3, 4]), w), *p).to_vector()
+        r, m = _both(naive, mine, fw)
+        assert r.shape == m.shape and norm_rel_err(m, r) <= 2e-6, p
+        def bw(d):
+            tx, tw = d.new_tensor_by_vector(S([7, 6, 3], 2), x), d.new_tensor_by_vector(S([3, 2, 3, 4]), w)
+            ty = d.conv2d_fw(tx, tw, *p)
+            gy = d.new_tensor_by_vector(ty.shape(), np.linspace(-1, 1, ty.shape().size()).astype(np.float32))
+            gx, gw = d.new_tensor_by_constant(tx.shape(), 0), d.new_tensor_by_constant(tw.shape(), 0)
+            d.conv2d_bw(tx, tw, ty, gy, *p, gx, gw)
+            return np.concatenate([gx.to_vector(), gw.to_vector()])
+        r, m = _both(naive, mine, bw)
+        assert norm_rel_err(m, r) <= 2e-6, p
+    for p in ((2, 2, 0, 0, 2, 2), (3, 2, 1, 1, 2, 1)):                          # window, padding, stride
+        def fw(d):
+            return d.max_pool2d_fw(d.new_tensor_by_vector(S([7, 6, 3], 2), x), *p).to_vector()
+        r, m = _both(naive, mine, fw)
+        assert np.array_equal(r, m), p
