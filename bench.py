@@ -532,6 +532,9 @@ def main():
         "vs_baseline": None, "dtype": "f32" if w.storage == "f32" else w.storage, "data": "synthetic",
         "config": {"workload": "%s: a,b,gy {%d,%d}x%d fp32, fw + both gradients"
                    % (head["workload"], w.di, w.dj, w.bs),
+                   "streams": "one (--in-order)" if args.in_order else
+                              "library default: a second stream for runs of independent matmul calls of at most 4 GFLOP "
+                              "(this workload's products are larger and run in order)",
                    "tolerance": "max|x-ref|/max|ref| <= %.0e vs CPU oracle" % w.tolerance},
         "frac_of_mfma_peak": head["frac_mfma_peak"],
         "roofline": roofline,
