@@ -533,8 +533,9 @@ def main():
         "config": {"workload": "%s: a,b,gy {%d,%d}x%d fp32, fw + both gradients"
                    % (head["workload"], w.di, w.dj, w.bs),
                    "streams": "one (--in-order)" if args.in_order else
-                              "library default: a second stream for runs of independent matmul calls of at most 4 GFLOP "
-                              "(this workload's products are larger and run in order)",
+                              "library default: a second stream for runs of independent matmul calls of at most 4 GFLOP (%s)"
+                              % ("this workload's products are larger and run in order" if w.flops_per_step() / 3 > 4e9
+                                 else "this workload's calls use it"),
                    "tolerance": "max|x-ref|/max|ref| <= %.0e vs CPU oracle" % w.tolerance},
         "frac_of_mfma_peak": head["frac_mfma_peak"],
         "roofline": roofline,
