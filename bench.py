@@ -36,11 +36,11 @@ HEADLINE = "square_batched"
 # y += x of known size in the same runs), summed over a step's launches ("HBM bytes per step by the
 # counters" there).  Algorithmic bytes for comparison are Workload.bytes_per_step().
 COUNTER_TRAFFIC_BYTES_PER_STEP = {
-    "square_batched": 762.6e6,       # 206.19 + 284.05 + 272.38 MB: the three gemm_f32_lds_kernel launches
-    "dense": 11.47e6,                # gemm_f32_direct_kernel 3.95 + gemm_f32_pair_kernel 7.52 MB
-    "rnn_gate": 872.3e6,             # 30 x (9.64 + 19.44 MB)
-    "output_projection": 4474.4e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.19 MB)
-    "half_storage": 6297.4e6,        # 2 x 2122.67 + 1984.86 + 67.17 MB (transposed copy of a)
+    "square_batched": 762.4e6,       # 206.14 + 283.93 + 272.32 MB: the three gemm_f32_lds_kernel launches
+    "dense": 14.58e6,                # gemm_f32_tile16_kernel 7.06 + gemm_f32_pair_kernel 7.52 MB
+    "rnn_gate": 872.4e6,             # 30 x (9.64 + 19.44 MB)
+    "output_projection": 4473.4e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.16 MB)
+    "half_storage": 6273.2e6,        # 2 x 2122.67 + 1960.7 + 67.17 MB (transposed copy of a)
 }
 # per launch of the headline kernel (average of its three operand-layout instantiations)
 HEADLINE_TRAFFIC_BYTES = COUNTER_TRAFFIC_BYTES_PER_STEP["square_batched"] / 3

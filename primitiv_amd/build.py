@@ -24,6 +24,7 @@ SOURCES = [
     "phip_random.hip",
     "phip_gemm_f32.hip",
     "phip_gemm_f32_direct.hip",
+    "phip_gemm_f32_tile16.hip",
     "phip_gemm_f32_lds.hip",
     "phip_gemm_f32_slab.hip",
     "phip_gemm_f32_rankk.hip",

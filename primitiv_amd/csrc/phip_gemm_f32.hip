@@ -58,6 +58,8 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   if (rc != PHIP_OK || handled) return rc;
   rc = gemm_f32_lds(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;
+  rc = gemm_f32_tile16(ctx, p, &handled);
+  if (rc != PHIP_OK || handled) return rc;
   rc = gemm_f32_direct(ctx, p, &handled);
   if (rc != PHIP_OK || handled) return rc;
   StagedPlan plan;

@@ -217,6 +217,7 @@ inline bool rows_aligned16(const void *ptr, int per16, long ld, long s = 0, long
 
 int gemm_f32(phip_ctx *ctx, const Gemm &g);
 int gemm_f32_direct(phip_ctx *ctx, const Gemm &g, bool *handled);
+int gemm_f32_tile16(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_lds(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_slab(phip_ctx *ctx, const Gemm &g, bool *handled);
 int gemm_f32_rankk(phip_ctx *ctx, const Gemm &g, bool *handled);

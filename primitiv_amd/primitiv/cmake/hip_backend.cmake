@@ -46,6 +46,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_random.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_direct.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_tile16.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_lds.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_slab.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_f32_rankk.hip

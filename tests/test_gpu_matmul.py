@@ -10,6 +10,7 @@ import pytest
 
 import oracle
 import primitiv_amd as pa
+from primitiv_amd import _lib
 from primitiv_amd.configs import WORKLOADS
 from util import norm_rel_err, np_matmul_bw, np_matmul_fw, vector_match
 
@@ -403,6 +404,35 @@ def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(first, oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)) <= F32_TOL
     for _ in range(25):
         assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), first)
+
+
+# an overwriting product with very few outputs and a K of 256..1024 runs on 16 x 16 tiles whose
+# eight wavefronts split K (no exchange between workgroups): the dense layer, ragged rows and
+# columns, K not a multiple of the 16 k of a load round or of four (4-byte loads of b), the shortest
+# and longest K it takes, a minibatch folded into the columns
+TILE16_F32 = [(256, 784, 1, 1, 128), (250, 700, 1, 1, 100), (33, 1024, 17, 1, 1), (16, 256, 16, 1, 1),
+              (100, 701, 1, 1, 50), (129, 999, 3, 1, 7), (7, 513, 5, 1, 1), (300, 1000, 1, 1, 40)]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", TILE16_F32)
+def test_few_outputs_long_k_forward_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di * 7 + dj)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    ta = dev.new_tensor_by_vector(pa.Shape([di, dj], ba), a)
+    tb = dev.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    want = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    first = dev.matmul_fw(ta, tb).to_vector()
+    assert norm_rel_err(first, want) <= F32_TOL
+    # every element, not only the largest: a row or column dropped at a ragged edge shows here
+    assert np.max(np.abs(np.asarray(first) - want)) <= 1e-4 * max(1.0, np.max(np.abs(want)))
+    for _ in range(5):                      # overwrites whatever the pool block held, same bits every time
+        assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), first)
+    # b at an address that is not 16-byte aligned: the same product through 4-byte loads of b
+    whole = dev.new_tensor_by_vector(pa.Shape([dj * dk * bb + 1]), np.concatenate([[0.0], b]).astype(np.float32))
+    y = dev.new_raw_tensor(pa.Shape([di, dk], bb))
+    _lib.call("phip_matmul_fw_f32", dev.ctx(), ta.handle(), whole.handle() + 4, y.mutable_handle(), di, dj, dk, ba, bb)
+    assert norm_rel_err(y.to_vector(), want) <= F32_TOL
 
 
 # accumulating products whose contraction is cut between workgroups: the dense layer's and the
