@@ -104,9 +104,10 @@ int gemm_f32_tile16(phip_ctx *ctx, const Gemm &p, bool *handled) {
   const long tiles32 = (long)((p.M + 31) / 32) * ((p.N + 31) / 32);
   const long tiles16 = (long)((p.M + 15) / 16) * ((p.N + 15) / 16);
   // worth it where 32 x 32 tiles would have to share their K range between workgroups, and where
-  // the smaller tiles still fit the chip at once (with more tiles than that - the recurrent gate's
-  // 2600 x 64 outputs make 652 - the smaller tiles' doubled operand traffic costs what the shorter
-  // chain of loads saves: 15.0 against 15.4 us per timestep in order, 9.8 against 9.2 on two lanes)
+  // the smaller tiles still fit the chip at once.  (A recurrent gate's forward product, 2048 x 64
+  // outputs with K = 512, already runs unsplit on 128 tiles of 32 x 32 with one round of loads;
+  // on 512 tiles of 16 x 16 the doubled operand traffic costs what the extra workgroups gain:
+  // 15.0 against 15.4 us per timestep in order, 9.8 against 9.2 with two products in flight.)
   if (tiles32 * 2 >= cus || tiles16 > 2L * cus) return PHIP_OK;
   Tile16Args d;
   d.g = problem_args(p);
