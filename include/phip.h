@@ -19,6 +19,12 @@
  *    the host.  In-order execution is what makes immediate reuse of a pool
  *    block safe (the reference relies on the same property of the CUDA null
  *    stream, primitiv/devices/cuda/ops/copy_tensor.cu:20-23).
+ *  - A context is driven by one host thread at a time, like a device object of
+ *    the reference (its devices keep unguarded per-object state too, e.g.
+ *    primitiv/devices/cuda/device.h:242-248); different contexts may be used
+ *    from different threads.  Only the pool entry points (phip_pool_alloc,
+ *    phip_pool_free, phip_pool_free_by_id, phip_pool_stats) take the context's
+ *    lock, because tensor handles may be released from any thread.
  *  - Element types: f32 = float, f16 = IEEE binary16, bf16 = bfloat16.  The
  *    16-bit variants store 16-bit values and always accumulate in fp32.
  */
@@ -125,10 +131,14 @@ int phip_free(phip_ctx *ctx, void *ptr);
  * (at least `2*sizeof(float)`, primitiv/internal/cuda/utils.h:337-342),
  * per-size free lists, one retry after releasing the reserved blocks.
  * bytes == 0 yields *out = NULL, *allocated = 0.  The library takes the scratch
- * memory of its own kernels from the same pool (partial tiles of split
- * products, unfolded images, a transposed 16-bit operand), so those blocks are
- * powers of two as well and stay cached until released; the retry releases
- * the idle blocks of every context on the GPU. */
+ * memory of its elementwise, reduction and convolution kernels from the same
+ * pool (unfolded images, partial reductions, index lists); the scratch of the
+ * matrix products (partial tiles of split products, a transposed 16-bit
+ * operand) comes from a second pool of the same policy whose blocks are never
+ * handed to a caller, because products may run on two streams (see
+ * phip_set_overlap) and a block is reused in stream order.  Blocks of both
+ * are powers of two and stay cached until released; the retry releases the
+ * idle blocks of every context on the GPU. */
 int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated);
 int phip_pool_free(phip_ctx *ctx, void *ptr);
 /* Same as phip_pool_free but addressed by context id; succeeds silently when
@@ -137,7 +147,7 @@ int phip_pool_free(phip_ctx *ctx, void *ptr);
  * (primitiv/core/memory_pool.h:22-35, test/cuda_device_test.cc:66-78). */
 int phip_pool_free_by_id(uint64_t ctx_id, void *ptr);
 int phip_pool_release_reserved(phip_ctx *ctx);
-/* Bytes currently handed out / held in free lists. */
+/* Bytes currently handed out / held in free lists, both pools of the context together. */
 int phip_pool_stats(phip_ctx *ctx, uint64_t *supplied_bytes, uint64_t *reserved_bytes);
 
 /* ---- copies ---------------------------------------------------------------
@@ -194,8 +204,13 @@ int phip_matmul_fw_bf16(phip_ctx *ctx, const void *a, const void *b, void *y,
 
 /* ---- matmul forward without any allocation ---------------------------------
  * No counterpart in the reference.  For callers that cannot allocate device
- * memory during the call: code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc.  Same arguments, kernels and result bits as
+ * memory during the call: tight serving loops, harnesses that forbid
+ * hipMalloc, code that is being captured into a HIP graph.  (Capture has two
+ * more conditions, which no test here exercises: the lanes switched off with
+ * phip_set_overlap(ctx, 0), since an engaged lane records and waits for an
+ * event, and one uncaptured call of the same shape beforehand, since the first
+ * use of a kernel on a context sets a function attribute.)
+ * Same arguments, kernels and result bits as
  * phip_matmul_fw_f32; a product whose K range is split between workgroups
  * keeps its partial tiles and tile counters in a fixed array inside the
  * library's device code (PHIP_NOALLOC_SCRATCH_BYTES per GPU, held until the

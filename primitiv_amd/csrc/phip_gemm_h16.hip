@@ -403,13 +403,13 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec_a, bool ve
   a.partial = nullptr;
   void *block = nullptr;
   if (splits > 1) {
-    const int rc = phip_pool_alloc(ctx, (size_t)(4L * p.M * p.N * p.batch * splits), &block, nullptr);
+    const int rc = scratch_alloc(ctx, (size_t)(4L * p.M * p.N * p.batch * splits), &block);
     if (rc != PHIP_OK) return rc;
     a.partial = static_cast<float *>(block);
   }
   const long grid = tiles * splits;
   if (grid > 0x7fffffffL) {
-    if (block) phip_pool_free(ctx, block);
+    if (block) scratch_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "matmul problem too large for one launch");
   }
 
@@ -430,7 +430,7 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec_a, bool ve
   } else if (p.a_kmajor && p.b_kmajor) {
     PHIP_LAUNCH(true, true);
   } else {
-    if (block) phip_pool_free(ctx, block);
+    if (block) scratch_free(ctx, block);
     return fail(PHIP_ERR_INVALID_ARGUMENT, "operand layout combination not used by matmul");
   }
 #undef PHIP_LAUNCH_V
@@ -442,7 +442,7 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec_a, bool ve
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((finish_split_h16_kernel<BF16>), dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream,
                        a.partial, a.C, p.M, p.N, p.ldc, p.sC, p.batch, (int)splits, a.accumulate);
-    phip_pool_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
+    scratch_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
   }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;

@@ -57,7 +57,12 @@ struct phip_ctx {
   hipStream_t stream = nullptr;
   hipDeviceProp_t prop;
   phip::Pool pool;
-  std::mutex mutex;  // guards `pool`
+  // Scratch of the matrix products (partial tiles of a split product, a transposed operand): blocks
+  // that no caller ever sees.  A block freed when its launches have been enqueued may be handed out
+  // again at once only to a launch on the same stream; a caller's tensor from `pool` can be written
+  // by a product on the other lane, so the two kinds of block never trade places.
+  phip::Pool scratch_pool;
+  std::mutex mutex;  // guards `pool` and `scratch_pool`
   // Kernels whose dynamic-LDS limit has been raised on this context's device
   // (one bit per kernel, see phip::raise_lds_limit).
   uint32_t lds_limit_raised = 0;
@@ -151,12 +156,13 @@ int lanes_place(phip_ctx *ctx, const MemRange *ranges, int n, bool may_overlap, 
 // Entries of phip_ctx::tile_tickets.
 constexpr int kTicketSlots = 65536;
 
-// Scratch memory of a launch (partial tiles of a split product, a padded copy of
-// a small operand): a pool block, or, during an allocation-free call, a piece of
-// the device's fixed scratch array (no allocation; fails with a message when the
-// call needs more than kFixedScratchBytes in total).  scratch_free returns a pool
-// block; the stream is in order, so the block may be reused behind the launches
-// that read it.  tile_tickets gives the zeroed per-tile counters that go with it.
+// Scratch memory of a matrix product (partial tiles of a split product, a transposed
+// operand): a block of the context's private scratch pool, or, during an
+// allocation-free call, a piece of the device's fixed scratch array (no allocation;
+// fails with a message when the call needs more than kFixedScratchBytes in total).
+// scratch_free returns a block to the scratch pool; the stream is in order, so the
+// block may be reused behind the launches that read it.  tile_tickets gives the
+// zeroed per-tile counters that go with it.
 constexpr size_t kFixedScratchBytes = 16u << 20;
 int scratch_alloc(phip_ctx *ctx, size_t bytes, void **out);
 void scratch_free(phip_ctx *ctx, void *ptr);

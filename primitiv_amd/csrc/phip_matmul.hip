@@ -89,14 +89,14 @@ static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, voi
   // on that is less than what the product gains.
   if (elem != Elem::F32 && ba == 1 && di >= 1024 && dj >= 1024 && di % 8 == 0 && dj % 8 == 0 &&
       (long)dk * bb >= 16384 && (long)di * dj * 2 < (1L << 31)) {
-    struct Block {  // back to the pool on every way out; the stream orders its reuse
+    struct Block {  // back to the scratch pool on every way out; the stream orders its reuse
       phip_ctx *ctx;
       void *ptr;
       ~Block() {
-        if (ptr) phip_pool_free(ctx, ptr);
+        if (ptr) scratch_free(ctx, ptr);
       }
     } at{ctx, nullptr};
-    rc = phip_pool_alloc(ctx, (size_t)di * dj * 2, &at.ptr, nullptr);
+    rc = scratch_alloc(ctx, (size_t)di * dj * 2, &at.ptr);
     if (rc != PHIP_OK) return rc;
     rc = elem == Elem::F16 ? phip_transpose_fw_f16(ctx, a, at.ptr, di, dj, 1)
                            : phip_transpose_fw_bf16(ctx, a, at.ptr, di, dj, 1);

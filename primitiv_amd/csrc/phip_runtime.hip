@@ -51,8 +51,11 @@ static int fixed_scratch_of(int device, unsigned char **out) {
   return PHIP_OK;
 }
 
+static int pool_alloc_from(phip_ctx *ctx, Pool &pool, size_t bytes, void **out, size_t *allocated);
+static int pool_free_locked(Pool &pool, void *ptr);
+
 int scratch_alloc(phip_ctx *ctx, size_t bytes, void **out) {
-  if (!ctx->fixed_mode) return phip_pool_alloc(ctx, bytes, out, nullptr);
+  if (!ctx->fixed_mode) return pool_alloc_from(ctx, ctx->scratch_pool, bytes, out, nullptr);
   *out = nullptr;
   const size_t start = (ctx->fixed_used + 255) / 256 * 256;
   if (bytes > kFixedScratchBytes || start > kFixedScratchBytes - bytes) {
@@ -69,7 +72,8 @@ void scratch_free(phip_ctx *ctx, void *ptr) {
   if (ptr == nullptr) return;
   const unsigned char *p = static_cast<const unsigned char *>(ptr);
   if (ctx->fixed_scratch && p >= ctx->fixed_scratch && p < ctx->fixed_scratch + kFixedTicketBytes + kFixedScratchBytes) return;
-  (void)phip_pool_free(ctx, ptr);
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  (void)pool_free_locked(ctx->scratch_pool, ptr);
 }
 
 uint32_t *tile_tickets(phip_ctx *ctx) {
@@ -84,12 +88,14 @@ static unsigned ceil_log2(uint64_t x) {
 
 static int release_reserved_locked(phip_ctx *ctx) {
   int rc = PHIP_OK;
-  for (auto &list : ctx->pool.reserved) {
-    while (!list.empty()) {
-      if (hipFree(list.back()) != hipSuccess) {
-        rc = fail(PHIP_ERR_RUNTIME, "hipFree failed while releasing pool blocks");
+  for (Pool *pool : {&ctx->pool, &ctx->scratch_pool}) {
+    for (auto &list : pool->reserved) {
+      while (!list.empty()) {
+        if (hipFree(list.back()) != hipSuccess) {
+          rc = fail(PHIP_ERR_RUNTIME, "hipFree failed while releasing pool blocks");
+        }
+        list.pop_back();
       }
-      list.pop_back();
     }
   }
   return rc;
@@ -109,13 +115,58 @@ static void release_reserved_on_device(int device) {
   }
 }
 
-static int pool_free_locked(phip_ctx *ctx, void *ptr) {
-  auto it = ctx->pool.supplied.find(ptr);
-  if (it == ctx->pool.supplied.end()) {
+static int pool_free_locked(Pool &pool, void *ptr) {
+  auto it = pool.supplied.find(ptr);
+  if (it == pool.supplied.end()) {
     return fail(PHIP_ERR_INVALID_ARGUMENT, "Detected to dispose unknown handle: %p", ptr);
   }
-  ctx->pool.reserved[it->second].push_back(ptr);
-  ctx->pool.supplied.erase(it);
+  pool.reserved[it->second].push_back(ptr);
+  pool.supplied.erase(it);
+  return PHIP_OK;
+}
+
+// A block of at least `bytes` (rounded up to a power of two) from `pool`'s free lists or from hipMalloc.
+static int pool_alloc_from(phip_ctx *ctx, Pool &pool, size_t bytes, void **out, size_t *allocated) {
+  *out = nullptr;
+  if (allocated) *allocated = 0;
+  if (bytes == 0) return PHIP_OK;
+  if (bytes < Pool::kMinimumSize) bytes = Pool::kMinimumSize;
+  if (bytes > (1ull << 62)) {
+    return fail(PHIP_ERR_INVALID_ARGUMENT, "Invalid memory size: %zu", bytes);
+  }
+  const unsigned shift = ceil_log2(bytes);
+  const size_t block = 1ull << shift;
+  void *ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    auto &list = pool.reserved[shift];
+    if (!list.empty()) {
+      ptr = list.back();
+      list.pop_back();
+    }
+  }
+  if (ptr == nullptr) {
+    hipError_t e = hipMalloc(&ptr, block);
+    if (e != hipSuccess) {
+      // Most likely out of memory: give back every idle block of every context on this GPU (a fp32 and a
+      // 16-bit device object on one GPU each have a pool) and try again.
+      (void)hipGetLastError();
+      release_reserved_on_device(ctx->device);
+      e = hipMalloc(&ptr, block);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(e == hipErrorOutOfMemory ? PHIP_ERR_OUT_OF_MEMORY : PHIP_ERR_RUNTIME,
+                  "Memory allocation failed. Requested size: %zu (%s)", block,
+                  hipGetErrorString(e));
+    }
+  }
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    pool.supplied.emplace(ptr, shift);
+  }
+  *out = ptr;
+  if (allocated) *allocated = block;
   return PHIP_OK;
 }
 
@@ -218,10 +269,12 @@ int phip_ctx_destroy(phip_ctx *ctx) {
   {
     std::lock_guard<std::mutex> lock(ctx->mutex);
     // Blocks still handed out are freed too: handles may outlive the device.
-    for (auto &kv : ctx->pool.supplied) {
-      if (hipFree(kv.first) != hipSuccess) rc = fail(PHIP_ERR_RUNTIME, "hipFree failed");
+    for (phip::Pool *pool : {&ctx->pool, &ctx->scratch_pool}) {
+      for (auto &kv : pool->supplied) {
+        if (hipFree(kv.first) != hipSuccess) rc = fail(PHIP_ERR_RUNTIME, "hipFree failed");
+      }
+      pool->supplied.clear();
     }
-    ctx->pool.supplied.clear();
     int r2 = phip::release_reserved_locked(ctx);
     if (r2 != PHIP_OK) rc = r2;
   }
@@ -325,54 +378,14 @@ int phip_free(phip_ctx *ctx, void *ptr) {
 int phip_pool_alloc(phip_ctx *ctx, size_t bytes, void **out, size_t *allocated) {
   PHIP_ENTER_HOST(ctx);
   PHIP_REQUIRE(out != nullptr, "null output pointer");
-  *out = nullptr;
-  if (allocated) *allocated = 0;
-  if (bytes == 0) return PHIP_OK;
-  if (bytes < phip::Pool::kMinimumSize) bytes = phip::Pool::kMinimumSize;
-  if (bytes > (1ull << 62)) {
-    return fail(PHIP_ERR_INVALID_ARGUMENT, "Invalid memory size: %zu", bytes);
-  }
-  const unsigned shift = phip::ceil_log2(bytes);
-  const size_t block = 1ull << shift;
-  void *ptr = nullptr;
-  {
-    std::lock_guard<std::mutex> lock(ctx->mutex);
-    auto &list = ctx->pool.reserved[shift];
-    if (!list.empty()) {
-      ptr = list.back();
-      list.pop_back();
-    }
-  }
-  if (ptr == nullptr) {
-    hipError_t e = hipMalloc(&ptr, block);
-    if (e != hipSuccess) {
-      // Most likely out of memory: give back every idle block of every context on this GPU (a fp32 and a
-      // 16-bit device object on one GPU each have a pool) and try again.
-      (void)hipGetLastError();
-      phip::release_reserved_on_device(ctx->device);
-      e = hipMalloc(&ptr, block);
-    }
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      return fail(e == hipErrorOutOfMemory ? PHIP_ERR_OUT_OF_MEMORY : PHIP_ERR_RUNTIME,
-                  "Memory allocation failed. Requested size: %zu (%s)", block,
-                  hipGetErrorString(e));
-    }
-  }
-  {
-    std::lock_guard<std::mutex> lock(ctx->mutex);
-    ctx->pool.supplied.emplace(ptr, shift);
-  }
-  *out = ptr;
-  if (allocated) *allocated = block;
-  return PHIP_OK;
+  return phip::pool_alloc_from(ctx, ctx->pool, bytes, out, allocated);
 }
 
 int phip_pool_free(phip_ctx *ctx, void *ptr) {
   PHIP_REQUIRE(ctx != nullptr, "null context");
   if (ptr == nullptr) return PHIP_OK;
   std::lock_guard<std::mutex> lock(ctx->mutex);
-  return phip::pool_free_locked(ctx, ptr);
+  return phip::pool_free_locked(ctx->pool, ptr);
 }
 
 int phip_pool_free_by_id(uint64_t ctx_id, void *ptr) {
@@ -381,7 +394,7 @@ int phip_pool_free_by_id(uint64_t ctx_id, void *ptr) {
   auto it = phip::g_registry.find(ctx_id);
   if (it == phip::g_registry.end()) return PHIP_OK;  // pool already gone
   std::lock_guard<std::mutex> lock(it->second->mutex);
-  return phip::pool_free_locked(it->second, ptr);
+  return phip::pool_free_locked(it->second->pool, ptr);
 }
 
 int phip_pool_release_reserved(phip_ctx *ctx) {
@@ -400,9 +413,11 @@ int phip_pool_stats(phip_ctx *ctx, uint64_t *supplied_bytes, uint64_t *reserved_
   PHIP_REQUIRE(ctx != nullptr, "null context");
   std::lock_guard<std::mutex> lock(ctx->mutex);
   uint64_t s = 0, r = 0;
-  for (auto &kv : ctx->pool.supplied) s += 1ull << kv.second;
-  for (size_t i = 0; i < ctx->pool.reserved.size(); ++i) {
-    r += (1ull << i) * ctx->pool.reserved[i].size();
+  for (const phip::Pool *pool : {&ctx->pool, &ctx->scratch_pool}) {
+    for (auto &kv : pool->supplied) s += 1ull << kv.second;
+    for (size_t i = 0; i < pool->reserved.size(); ++i) {
+      r += (1ull << i) * pool->reserved[i].size();
+    }
   }
   if (supplied_bytes) *supplied_bytes = s;
   if (reserved_bytes) *reserved_bytes = r;

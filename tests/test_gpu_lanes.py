@@ -305,3 +305,38 @@ def test_gradients_reset_between_calls_as_a_backward_pass_does():
                 assert norm_rel_err(got, want) <= 1e-5
     _, gb = oracle.matmul_bw(a, bs[1], gys[1], np.zeros(m * k, np.float32), np.zeros(k * n, np.float32), m, k, n, 1, 1)
     assert norm_rel_err(results[1][0], gb) <= 1e-4      # timestep 5 uses operands 5 % 4 = 1
+
+
+def test_scratch_of_a_split_product_never_becomes_a_tensor_of_the_other_lane():
+    # A forward product with few output tiles and a long K meets through partial tiles in scratch
+    # memory, which goes back to its pool when the launch has been enqueued.  The outputs allocated
+    # next cover every power-of-two size class that scratch block can have, and their products have
+    # operands of their own, so they run on the other lane: if a scratch block could come back as one
+    # of them, it would be overwritten under the first product.  Also the other way round: tensors
+    # released while a product on the other lane may still read them.
+    m, k, n = 96, 4000, 15
+    rng = np.random.default_rng(8)
+    a = rng.standard_normal(m * k).astype(np.float32) / np.sqrt(k)
+    b = rng.standard_normal(k * n).astype(np.float32)
+    small_a = rng.standard_normal(64 * 8).astype(np.float32)
+    classes = [1 << s for s in range(12, 23)]               # 4 KiB ... 4 MiB outputs
+    small_b = {c: rng.standard_normal(8 * (c // 256)).astype(np.float32) for c in classes}
+
+    def program(d):
+        ta, tb = d.new_tensor_by_vector(S([m, k]), a), d.new_tensor_by_vector(S([k, n]), b)
+        tsa = d.new_tensor_by_vector(S([64, 8]), small_a)
+        tsb = {c: d.new_tensor_by_vector(S([8, c // 256]), small_b[c]) for c in classes}
+        outs = []
+        for it in range(6):
+            y = d.matmul_fw(ta, tb)                          # split: partial tiles in scratch
+            fresh = [d.matmul_fw(tsa, tsb[c]) for c in classes]   # new outputs of every class, other operands
+            y2 = d.matmul_fw(ta, tb)                         # again, while the small products are in flight
+            outs += [y.to_vector(), y2.to_vector(), fresh[it % len(fresh)].to_vector()]
+            del fresh                                        # blocks back to the pool for the next round
+        return outs
+
+    lanes, in_order = _run_both(program)
+    _same_bits(lanes, in_order)
+    want = oracle.matmul_fw(a, b, m, k, n, 1, 1)
+    for i in range(0, len(in_order), 3):
+        assert norm_rel_err(lanes[i], want) <= 1e-4 and norm_rel_err(lanes[i + 1], want) <= 1e-4

@@ -24,12 +24,13 @@ F32_TOL = 1e-4
 
 # (di, dj, dk, ba, bb): products whose K range is cut between workgroups (partial
 # tiles + tile counters in scratch), the output projection's forward product (a
-# padded copy of x in scratch) and an unsplit one.
+# launch that mixes whole tiles with tiles cut in K ranges: partial tiles of the
+# latter in scratch) and an unsplit one.
 SEQUENCE = [
     (2048, 512, 1, 1, 64),     # recurrent gate forward
     (256, 784, 1, 1, 128),     # dense forward: smaller, right after the larger one
     (96, 1000, 5, 1, 3),       # ragged, split
-    (10000, 650, 1, 1, 64),    # streamed operand, x padded into scratch
+    (10000, 650, 1, 1, 64),    # streamed operand: whole tiles beside split ones
     (1024, 4096, 512, 1, 1),   # mid-size, long K: large tiles, K cut in 8: exactly 16 MiB of partial tiles
     (768, 4096, 96, 1, 1),     # few tiles, long K
     (200, 3000, 40, 2, 2),     # per-sample products, split
