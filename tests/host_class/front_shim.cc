@@ -544,6 +544,89 @@ int hc_scenario_xor_training_step(Device *dev, float eta, float *values, float *
   HC_END
 }
 
+// One LSTM step with primitiv's own Graph on `dev`, written as the reference's graph tests write it
+// (test/graph_test.cc:437-551 CheckLSTM with eight weight matrices and four biases when `stacked`
+// is 0, :553-646 CheckConcatLSTM with stacked weights and slices otherwise).  `params` holds the
+// parameters' initial values in the order the test declares them (40 floats either way).
+//   losses: the 4 values of the loss node;  sum_loss: batch::sum(sum(loss, 0));
+//   num_operators: what the graph counts;  grads: the parameters' gradients, same order as `params`.
+int hc_scenario_lstm_step(Device *dev, int stacked, const float *params, const float *x_values, const float *h_values,
+                          float *losses, float *sum_loss, U32 *num_operators, float *grads) {
+  HC_TRY
+  namespace F = primitiv::functions;
+  using primitiv::Node;
+  using primitiv::Parameter;
+  Device::set_default(*dev);
+  std::vector<Parameter *> ps;
+  auto make = [&](const Shape &shape) {
+    const U32 n = shape.size();
+    ps.push_back(new Parameter(shape, std::vector<float>(params, params + n)));
+    params += n;
+    return ps.back();
+  };
+  struct Cleanup {
+    std::vector<Parameter *> &v;
+    ~Cleanup() { for (Parameter *p : v) delete p; }
+  } cleanup{ps};
+
+  primitiv::Graph g;
+  primitiv::Graph::set_default(g);
+  Node loss_node, total;
+  const std::vector<float> xv(x_values, x_values + 4), hv(h_values, h_values + 4);
+  if (!stacked) {
+    for (int k = 0; k < 8; ++k) make(Shape({2, 2}));
+    for (int k = 0; k < 4; ++k) make(Shape({2}));
+    for (Parameter *p : ps) p->reset_gradient();
+    const Node x = F::input<Node>(Shape({2}, 2), xv);
+    const Node h = F::input<Node>(Shape({2}, 2), hv);
+    const Node c = F::zeros<Node>({2});
+    std::vector<Node> n;
+    for (Parameter *p : ps) n.push_back(F::parameter<Node>(*p));
+    const Node i = F::sigmoid(F::matmul(n[0], x) + F::matmul(n[4], h) + n[8]);
+    const Node f = F::sigmoid(F::matmul(n[1], x) + F::matmul(n[5], h) + n[9]);
+    const Node o = F::sigmoid(F::matmul(n[2], x) + F::matmul(n[6], h) + n[10]);
+    const Node j = F::tanh(F::matmul(n[3], x) + F::matmul(n[7], h) + n[11]);
+    const Node cc = f * c + i * j;
+    const Node hh = o * F::tanh(cc);
+    const Node t = F::zeros<Node>({2});
+    const Node diff = hh - t;
+    loss_node = diff * diff;
+    total = F::batch::sum(F::sum(loss_node, 0));
+  } else {
+    make(Shape({8, 2}));
+    make(Shape({8, 2}));
+    make(Shape({8}));
+    for (Parameter *p : ps) p->reset_gradient();
+    const Node x = F::input<Node>(Shape({2}, 2), xv);
+    const Node h = F::input<Node>(Shape({2}, 2), hv);
+    const Node c = F::zeros<Node>({2});
+    const Node Wx = F::parameter<Node>(*ps[0]);
+    const Node Wh = F::parameter<Node>(*ps[1]);
+    const Node b = F::parameter<Node>(*ps[2]);
+    const Node u = F::matmul(Wx, x) + F::matmul(Wh, h) + b;
+    const Node i = F::sigmoid(F::slice(u, 0, 0, 2));
+    const Node f = F::sigmoid(F::slice(u, 0, 2, 4));
+    const Node o = F::sigmoid(F::slice(u, 0, 4, 6));
+    const Node j = F::tanh(F::slice(u, 0, 6, 8));
+    const Node cc = f * c + i * j;
+    const Node hh = o * F::tanh(cc);
+    const Node t = F::zeros<Node>({2});
+    const Node diff = hh - t;
+    loss_node = diff * diff;
+    total = F::batch::sum(F::sum(loss_node, 0));
+  }
+  *num_operators = g.num_operators();
+  const std::vector<float> lv = g.forward(loss_node).to_vector();
+  std::copy(lv.begin(), lv.end(), losses);
+  *sum_loss = g.forward(total).to_float();
+  total.backward();
+  for (Parameter *p : ps) {
+    const std::vector<float> v = p->gradient().to_vector();
+    grads = std::copy(v.begin(), v.end(), grads);
+  }
+  HC_END
+}
+
 // Copies between a host device of the reference and `dev`, both ways (test/tensor_forward_test.cc:67-84):
 // out receives the values after naive -> dev -> naive.
 int hc_scenario_copy_through_naive(Device *dev, const float *values, U32 n, float *out) {

@@ -2,10 +2,14 @@
 reference's graph test (test/graph_test.cc:362-435, every node value is a
 golden vector there), forward and backward, op by op as primitiv's graph
 would call the device."""
+import json
+import os
+
 import numpy as np
 import pytest
 
 import primitiv_amd as pa
+from graph_tape import Tape
 
 pytestmark = pytest.mark.gpu
 
@@ -183,3 +187,131 @@ def test_small_convolutional_network_against_oracle(dev):
     rg_x, rg_w1 = oracle.conv2d_bw(x, w1, g_c1.to_vector(), z(x.size), z(w1.size), [12, 12, 1], bs, [3, 3, 1, 4], 1, *conv)
     near(g_x, rg_x, "g_x")
     near(g_w1, rg_w1, "g_w1")
+
+
+# ---- the reference's two LSTM graph tests (test/graph_test.cc:437-551, 553-646) -----------------
+#
+# Both build one LSTM step on a minibatch of two, loss = sum of squares of the new hidden state:
+# CheckLSTM with eight weight matrices and four biases, CheckConcatLSTM with the gates' weights
+# stacked and `slice` to take the gates apart ("all values and gradients should be same").  What
+# the tests hold as numbers - parameters, inputs, operator count and the four losses at 1e-6 - is in
+# tests/golden/graph_vectors.json (written from the test's text by extract_graph_vectors.py).
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "graph_vectors.json")) as _f:
+    GRAPH_VECTORS = json.load(_f)
+
+
+def _lstm_float64(case):
+    """Values and gradients of the stacked-weights LSTM step in float64 (closed form of one step)."""
+    P = case["parameters"]
+    col = lambda p: np.asarray(p["values"], dtype=np.float64).reshape(p["shape"][::-1]).T     # column-major
+    Wx, Wh, b = col(P["pWx"]), col(P["pWh"]), np.asarray(P["pb"]["values"], dtype=np.float64)
+    X = np.asarray(case["inputs"]["x"]["values"], dtype=np.float64).reshape(2, 2)          # samples x inputs
+    H = np.asarray(case["inputs"]["h"]["values"], dtype=np.float64).reshape(2, 2)
+    sig = lambda v: 1 / (1 + np.exp(-v))
+    U = X @ Wx.T + H @ Wh.T + b                                                               # samples x 8
+    i, f, o, j = sig(U[:, 0:2]), sig(U[:, 2:4]), sig(U[:, 4:6]), np.tanh(U[:, 6:8])
+    c = np.zeros(2)
+    cc = f * c + i * j
+    hh = o * np.tanh(cc)
+    loss = hh * hh
+    dhh = 2 * hh
+    do, dcc = dhh * np.tanh(cc), dhh * o * (1 - np.tanh(cc) ** 2)
+    di, dj, df = dcc * j, dcc * i, dcc * c
+    dU = np.concatenate([di * i * (1 - i), df * f * (1 - f), do * o * (1 - o), dj * (1 - j ** 2)], axis=1)
+    return {"loss": loss.reshape(-1), "i": i, "f": f, "o": o, "j": j, "cc": cc, "hh": hh,
+            "gWx": dU.T @ X, "gWh": dU.T @ H, "gb": dU.sum(axis=0), "gx": dU @ Wx, "gh": dU @ Wh,
+            "gc": (dcc * f).sum(axis=0)}
+
+
+def _colmajor(m):
+    return np.asarray(m).T.reshape(-1)
+
+
+def _lstm_tolerances(dev):
+    f32 = dev._SUFFIX == "f32"
+    # fp32: the reference's own bound on the losses.  16-bit storage: every node value is rounded to
+    # 11 (fp16) or 8 (bf16) significant bits; the losses are squares of values around 0.05 - 0.17.
+    return (1e-6, 2e-6) if f32 else ((1e-3, 2e-2) if dev._SUFFIX == "f16" else (4e-3, 5e-2))
+
+
+def test_lstm_with_separate_gate_weights(dev):
+    case, ref = GRAPH_VECTORS["CheckLSTM"], _lstm_float64(GRAPH_VECTORS["CheckConcatLSTM"])
+    loss_tol, grad_tol = _lstm_tolerances(dev)
+    S, P = pa.Shape, case["parameters"]
+    g = Tape(dev)
+    x = g.input(S(case["inputs"]["x"]["shape"], 2), case["inputs"]["x"]["values"])
+    h = g.input(S(case["inputs"]["h"]["shape"], 2), case["inputs"]["h"]["values"])
+    c = g.constant(S([2]), 0)
+    names = ["pWix", "pWfx", "pWox", "pWjx", "pWih", "pWfh", "pWoh", "pWjh", "pbi", "pbf", "pbo", "pbj"]
+    n = {k: g.input(S(P[k]["shape"]), P[k]["values"]) for k in names}       # parameter nodes, in the test's order
+
+    def gate(act, wx, wh, b):
+        return act(g.add(g.add(g.matmul(n[wx], x), g.matmul(n[wh], h)), n[b]))
+
+    i = gate(g.sigmoid, "pWix", "pWih", "pbi")
+    f = gate(g.sigmoid, "pWfx", "pWfh", "pbf")
+    o = gate(g.sigmoid, "pWox", "pWoh", "pbo")
+    j = gate(g.tanh, "pWjx", "pWjh", "pbj")
+    cc = g.add(g.multiply(f, c), g.multiply(i, j))
+    hh = g.multiply(o, g.tanh(cc))
+    t = g.constant(S([2]), 0)
+    diff = g.subtract(hh, t)
+    loss = g.multiply(diff, diff)
+    sum_loss = g.batch_sum(g.sum(loss, 0))
+    assert g.num_operators() == case["num_operators"] == 45
+
+    want = np.asarray(case["expected_losses"], dtype=np.float32)
+    assert np.allclose(g.value(loss).to_vector(), want, rtol=0, atol=loss_tol)
+    assert abs(g.value(sum_loss).to_float() - float(want.sum())) <= 4 * loss_tol
+    assert np.allclose(ref["loss"], want, rtol=0, atol=1e-7)                # the float64 closed form agrees with the test
+    for node, key in ((i, "i"), (f, "f"), (o, "o"), (j, "j"), (cc, "cc"), (hh, "hh")):
+        assert np.allclose(g.value(node).to_vector(), ref[key].reshape(-1), rtol=0, atol=max(loss_tol, grad_tol / 4)), key
+
+    g.backward(sum_loss)
+    rows = {"i": slice(0, 2), "f": slice(2, 4), "o": slice(4, 6), "j": slice(6, 8)}
+    for gate_name, r in rows.items():
+        assert np.allclose(g.gradient(n["pW%sx" % gate_name]).to_vector(), _colmajor(ref["gWx"][r]), rtol=0, atol=grad_tol)
+        assert np.allclose(g.gradient(n["pW%sh" % gate_name]).to_vector(), _colmajor(ref["gWh"][r]), rtol=0, atol=grad_tol)
+        assert np.allclose(g.gradient(n["pb%s" % gate_name]).to_vector(), ref["gb"][r], rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(x).to_vector(), ref["gx"].reshape(-1), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(h).to_vector(), ref["gh"].reshape(-1), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(c).to_vector(), ref["gc"], rtol=0, atol=grad_tol)
+
+
+def test_lstm_with_stacked_gate_weights(dev):
+    case = GRAPH_VECTORS["CheckConcatLSTM"]
+    ref = _lstm_float64(case)
+    loss_tol, grad_tol = _lstm_tolerances(dev)
+    S, P = pa.Shape, case["parameters"]
+    g = Tape(dev)
+    x = g.input(S(case["inputs"]["x"]["shape"], 2), case["inputs"]["x"]["values"])
+    h = g.input(S(case["inputs"]["h"]["shape"], 2), case["inputs"]["h"]["values"])
+    c = g.constant(S([2]), 0)
+    Wx, Wh, b = (g.input(S(P[k]["shape"]), P[k]["values"]) for k in ("pWx", "pWh", "pb"))
+    u = g.add(g.add(g.matmul(Wx, x), g.matmul(Wh, h)), b)
+    i = g.sigmoid(g.slice(u, 0, 0, 2))
+    f = g.sigmoid(g.slice(u, 0, 2, 4))
+    o = g.sigmoid(g.slice(u, 0, 4, 6))
+    j = g.tanh(g.slice(u, 0, 6, 8))
+    cc = g.add(g.multiply(f, c), g.multiply(i, j))
+    hh = g.multiply(o, g.tanh(cc))
+    t = g.constant(S([2]), 0)
+    diff = g.subtract(hh, t)
+    loss = g.multiply(diff, diff)
+    sum_loss = g.batch_sum(g.sum(loss, 0))
+    assert g.num_operators() == case["num_operators"] == 28
+
+    want = np.asarray(case["expected_losses"], dtype=np.float32)
+    assert np.allclose(g.value(loss).to_vector(), want, rtol=0, atol=loss_tol)
+    assert abs(g.value(sum_loss).to_float() - float(want.sum())) <= 4 * loss_tol
+    for node, key in ((i, "i"), (f, "f"), (o, "o"), (j, "j"), (cc, "cc"), (hh, "hh")):
+        assert np.allclose(g.value(node).to_vector(), ref[key].reshape(-1), rtol=0, atol=max(loss_tol, grad_tol / 4)), key
+
+    g.backward(sum_loss)
+    assert np.allclose(g.gradient(Wx).to_vector(), _colmajor(ref["gWx"]), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(Wh).to_vector(), _colmajor(ref["gWh"]), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(b).to_vector(), ref["gb"], rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(x).to_vector(), ref["gx"].reshape(-1), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(h).to_vector(), ref["gh"].reshape(-1), rtol=0, atol=grad_tol)
+    assert np.allclose(g.gradient(c).to_vector(), ref["gc"], rtol=0, atol=grad_tol)

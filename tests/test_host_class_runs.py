@@ -402,3 +402,41 @@ def test_xor_perceptron_op_by_op(anydev):
     import test_gpu_graph
     test_gpu_graph.test_xor_perceptron_forward_and_backward(anydev)
     test_gpu_graph.test_matmul_gradients_of_one_tensor_used_twice(anydev)
+
+
+def test_lstm_graphs_op_by_op(anydev):
+    # test/graph_test.cc:437-646 through Device's front, operator by operator
+    import test_gpu_graph
+    test_gpu_graph.test_lstm_with_separate_gate_weights(anydev)
+    test_gpu_graph.test_lstm_with_stacked_gate_weights(anydev)
+
+
+@pytest.mark.parametrize("stacked", [0, 1])
+def test_lstm_graphs_with_the_reference_graph(anydev, stacked):
+    # the same two tests built with primitiv's own Graph / Node / Parameter on devices::HIP:
+    # operator count, the four golden losses at the test's 1e-6, gradients against float64
+    import test_gpu_graph as tg
+    case = tg.GRAPH_VECTORS["CheckConcatLSTM" if stacked else "CheckLSTM"]
+    ref = tg._lstm_float64(tg.GRAPH_VECTORS["CheckConcatLSTM"])
+    order = (["pWx", "pWh", "pb"] if stacked else
+             ["pWix", "pWfx", "pWox", "pWjx", "pWih", "pWfh", "pWoh", "pWjh", "pbi", "pbf", "pbo", "pbj"])
+    params = np.concatenate([np.asarray(case["parameters"][k]["values"], dtype=np.float32) for k in order])
+    x = np.asarray(case["inputs"]["x"]["values"], dtype=np.float32)
+    h = np.asarray(case["inputs"]["h"]["values"], dtype=np.float32)
+    losses, grads = np.zeros(4, np.float32), np.zeros(40, np.float32)
+    total, nops = ctypes.c_float(0), ctypes.c_uint32(0)
+    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    hc.call("hc_scenario_lstm_step", anydev.ptr, stacked, vp(params), vp(x), vp(h), vp(losses), ctypes.byref(total),
+            ctypes.byref(nops), vp(grads))
+    assert nops.value == case["num_operators"]
+    loss_tol, grad_tol = tg._lstm_tolerances(anydev)
+    want = np.asarray(case["expected_losses"], dtype=np.float32)
+    assert np.allclose(losses, want, rtol=0, atol=loss_tol)
+    assert abs(total.value - float(want.sum())) <= 4 * loss_tol
+    if stacked:
+        G = np.concatenate([tg._colmajor(ref["gWx"]), tg._colmajor(ref["gWh"]), ref["gb"]])
+    else:
+        rows = [slice(0, 2), slice(2, 4), slice(4, 6), slice(6, 8)]
+        G = np.concatenate([tg._colmajor(ref["gWx"][r]) for r in rows] + [tg._colmajor(ref["gWh"][r]) for r in rows] +
+                           [ref["gb"][r] for r in rows])
+    assert np.allclose(grads, G, rtol=0, atol=grad_tol)
