@@ -31,6 +31,7 @@ from primitiv_amd.configs import WORKLOADS  # noqa: E402
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2516.6, "bf16": 2516.6}
 PEAK_HBM_GBS = 8000.0
 HEADLINE = "square_batched"
+STORAGE_CODE = {"f32": 0, "f16": 1, "bf16": 2}
 # HBM bytes per step by rocprofv3's counters, from profiles/matmul_workloads_kernel_times_traffic_counters.txt
 # section 2: per dispatch FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB (the factors read off a streaming
 # y += x of known size in the same runs), summed over a step's launches ("HBM bytes per step by the
@@ -44,6 +45,22 @@ COUNTER_TRAFFIC_BYTES_PER_STEP = {
 }
 # per launch of the headline kernel (average of its three operand-layout instantiations)
 HEADLINE_TRAFFIC_BYTES = COUNTER_TRAFFIC_BYTES_PER_STEP["square_batched"] / 3
+# Workloads whose products are small enough for the library's second lane (at most 4 GFLOP each): the
+# step of record is taken with every launch on one stream, which is what a graph with other operations
+# between its products sees; the figure with independent calls on two lanes is reported beside it.
+PER_TIMESTEP = ("dense", "rnn_gate", "output_projection")
+
+NATIVE_SRC = os.path.join(ROOT, "bench_native.cc")
+NATIVE_LIB = os.path.join(ROOT, "libphip_bench.so")
+
+
+def build_native():
+    """Compiles the native timing loops (bench_native.cc, host code) against libphip.so."""
+    import subprocess
+    lib_dir = os.path.join(ROOT, "primitiv_amd")
+    subprocess.check_call(["g++", "-O2", "-std=c++11", "-fPIC", "-shared", "-Wall", "-Wextra", NATIVE_SRC, "-o",
+                           NATIVE_LIB, "-L" + lib_dir, "-lphip", "-Wl,-rpath,$ORIGIN/primitiv_amd"])
+    return NATIVE_LIB
 
 
 class Resident:
@@ -52,6 +69,7 @@ class Resident:
     def __init__(self, dev, w, seed=0):
         self.dev, self.w = dev, w
         a, bs, gys = w.inputs(seed=seed)
+        self.host = (a, bs, gys)
         S = pa.Shape
         self.a = dev.new_tensor_by_vector(S([w.di, w.dj], w.ba), a)
         self.b = [dev.new_tensor_by_vector(S([w.dj, w.dk], w.bb), x) for x in bs]
@@ -83,26 +101,92 @@ class Resident:
 # 3 warm-up steps of 0.9 ms, 122 behind 10, 129.6 behind 30 or 100): the untimed warm-up is the
 # requested number of steps and at least this much time.
 WARMUP_MIN_SECONDS = 0.06
+# "Sustains": the two MFMA-bound workloads are also timed over at least this long a run of back-to-back steps.
+SUSTAINED_MIN_SECONDS = 1.0
 
 
-def _warm_up(dev, step, warmup):
-    t0 = time.perf_counter()
-    for _ in range(warmup):
-        step()
-    dev.sync()
-    while time.perf_counter() - t0 < WARMUP_MIN_SECONDS:
-        for _ in range(8):
-            step()
-        dev.sync()
+class _Dims(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint32) for n in ("di", "dj", "dk", "ba", "bb")]
 
 
-def time_gpu(dev, res, steps, warmup):
-    """(host seconds, event seconds) for `steps` steps."""
+class _LstmDims(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint32) for n in ("in_size", "hidden", "batch", "timesteps")]
+
+
+_bench_lib = None
+
+
+def _native():
+    """libphip_bench.so: the timing loops in native code (bench_native.cc)."""
+    global _bench_lib
+    if _bench_lib is None:
+        _lib.lib()
+        if not os.path.exists(NATIVE_LIB):
+            raise _lib.Error("libphip_bench.so is not built; run `python __graft_entry__.py` or bench.build_native()")
+        l = ctypes.CDLL(NATIVE_LIB)
+        vp, pp, i = ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int
+        out = [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+        # device pointers are 64-bit: without these ctypes would pass them as C ints
+        l.phip_bench_raw_loop.argtypes = [vp, i, i, vp, vp, pp, pp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
+        l.phip_bench_front_loop.argtypes = [vp, i, vp, vp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
+        l.phip_bench_lstm_loop.argtypes = [vp, i, ctypes.POINTER(_LstmDims), vp, vp, vp, vp, pp, pp, vp, vp, i, i, i] + out
+        l.phip_bench_raw_loop.restype = l.phip_bench_front_loop.restype = l.phip_bench_lstm_loop.restype = i
+        _bench_lib = l
+    return _bench_lib
+
+
+class Loops:
+    """The native loops over one resident workload: raw (the two entry points on preallocated
+    outputs) and front (what primitiv's Device front does around them per call: y from the pool,
+    the per-timestep gradient from the pool and zero-filled, both handed back;
+    primitiv/core/device.cc:20-24,268-301).  Each call returns milliseconds per step by the
+    events on the library's stream and by the host clock."""
+
+    def __init__(self, dev, res):
+        self.dev, self.res, w = dev, res, res.w
+        n = w.steps
+        arr = lambda ptrs: (ctypes.c_void_p * n)(*ptrs)
+        self.b, self.gy = arr([p[0] for p in res.ptrs]), arr([p[1] for p in res.ptrs])
+        self.y, self.gb = arr([p[2] for p in res.ptrs]), arr([p[3] for p in res.ptrs])
+        self.d = _Dims(w.di, w.dj, w.dk, w.ba, w.bb)
+        self.n, self.code = n, STORAGE_CODE[w.storage]
+
+    def raw(self, steps, warmup, which=0):
+        """which: 0 = forward and backward calls, 1 = forward only, 2 = backward only."""
+        ev, host = ctypes.c_float(), ctypes.c_double()
+        r = self.res
+        _lib.check(_native().phip_bench_raw_loop(self.dev.ctx(), self.code, which, r.a.handle(), r.ga.handle(), self.b, self.gy,
+                                                 self.y, self.gb, ctypes.byref(self.d), self.n, steps, warmup,
+                                                 ctypes.byref(ev), ctypes.byref(host)))
+        return ev.value / steps, host.value / steps
+
+    def front(self, steps, warmup):
+        ev, host = ctypes.c_float(), ctypes.c_double()
+        r = self.res
+        _lib.check(_native().phip_bench_front_loop(self.dev.ctx(), self.code, r.a.handle(), r.ga.handle(), self.b,
+                                                   self.gy, ctypes.byref(self.d), self.n, steps, warmup,
+                                                   ctypes.byref(ev), ctypes.byref(host)))
+        return ev.value / steps, host.value / steps
+
+    def settle(self, warmup):
+        """Untimed steps: the requested number and at least WARMUP_MIN_SECONDS.  Returns (steps, seconds)."""
+        t0, done = time.perf_counter(), 0
+        if warmup:
+            self.raw(warmup, 0)
+            done = warmup
+        while time.perf_counter() - t0 < WARMUP_MIN_SECONDS:
+            self.raw(8, 0)
+            done += 8
+        return done, time.perf_counter() - t0
+
+
+def time_python_loop(dev, res, steps):
+    """Milliseconds per step (events, host clock) of the same calls issued by the interpreter."""
     ctx = dev.ctx()
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     _lib.call("phip_event_create", ctx, ctypes.byref(e0))
     _lib.call("phip_event_create", ctx, ctypes.byref(e1))
-    _warm_up(dev, res.step, warmup)
+    dev.sync()
     t0 = time.perf_counter()
     _lib.call("phip_event_record", ctx, e0)
     for _ in range(steps):
@@ -114,153 +198,157 @@ def time_gpu(dev, res, steps, warmup):
     _lib.call("phip_event_elapsed_ms", e0, e1, ctypes.byref(ms))
     _lib.call("phip_event_destroy", e0)
     _lib.call("phip_event_destroy", e1)
-    return host, ms.value * 1e-3
+    return ms.value / steps, host / steps * 1e3
 
 
-class _Dims(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_uint32) for n in ("di", "dj", "dk", "ba", "bb")]
+def _rel(x, ref):
+    return float(np.max(np.abs(np.asarray(x, dtype=np.float64) - ref)) / np.max(np.abs(ref)))
 
 
-_bench_lib = None
-
-
-def _native():
-    """libphip_bench.so: the same loops in native code (primitiv_amd/bench_front.cc)."""
-    global _bench_lib
-    if _bench_lib is None:
-        _lib.lib()
-        path = os.path.join(ROOT, "primitiv_amd", "libphip_bench.so")
-        if not os.path.exists(path):
-            raise _lib.Error("libphip_bench.so is not built; run `python -m primitiv_amd.build`")
-        l = ctypes.CDLL(path)
-        vp, pp, i = ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int
-        out = [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
-        # device pointers are 64-bit: without these ctypes would pass them as C ints
-        l.phip_bench_raw_loop.argtypes = [vp, vp, vp, pp, pp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
-        l.phip_bench_front_loop.argtypes = [vp, vp, vp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
-        l.phip_bench_raw_loop.restype = l.phip_bench_front_loop.restype = i
-        _bench_lib = l
-    return _bench_lib
-
-
-def time_front(dev, res, steps, warmup):
-    """Per-step milliseconds of the fp32 workload `res` in native loops: the two entry points on
-    preallocated outputs ("raw", what the Python loop above times), and with what primitiv's Device
-    front does around them per call ("front": y from the pool, the per-timestep gradient from the pool
-    and zero-filled, both handed back; primitiv/core/device.cc:20-24,268-301)."""
-    w = res.w
-    n = w.steps
-    arr = lambda ptrs: (ctypes.c_void_p * n)(*ptrs)
-    b, gy = arr([p[0] for p in res.ptrs]), arr([p[1] for p in res.ptrs])
-    y, gb = arr([p[2] for p in res.ptrs]), arr([p[3] for p in res.ptrs])
-    d = _Dims(w.di, w.dj, w.dk, w.ba, w.bb)
-    ev, host = ctypes.c_float(), ctypes.c_double()
-    out = {}
-    L = _native()
-    _lib.check(L.phip_bench_raw_loop(dev.ctx(), res.a.handle(), res.ga.handle(), b, gy, y, gb, ctypes.byref(d), n,
-                                     steps, warmup, ctypes.byref(ev), ctypes.byref(host)))
-    out["ms_per_step_native_raw"] = ev.value / steps
-    out["ms_per_step_native_raw_host_clock"] = host.value / steps
-    _lib.check(L.phip_bench_front_loop(dev.ctx(), res.a.handle(), res.ga.handle(), b, gy, ctypes.byref(d), n,
-                                       steps, warmup, ctypes.byref(ev), ctypes.byref(host)))
-    out["ms_per_step_front"] = ev.value / steps
-    out["ms_per_step_front_host_clock"] = host.value / steps
-    return out
-
-
-def cpu_baseline(w, threads=1):
-    """Times the CPU oracle (a port of the reference's Eigen device, one
-    thread, as the reference builds Eigen without OpenMP) on a bounded sample
-    of the workload and scales to TFLOP/s."""
+def cpu_baseline(w, res, threads=1):
+    """The CPU leg.  Times the CPU oracle (a port of the reference's Eigen device, one thread, as the
+    reference builds Eigen without OpenMP) on a bounded sample of the workload's own seeded inputs
+    and scales to TFLOP/s; and uses the same oracle as the checker of this run's timed buffers:
+    the forward result that the timed loop left on the device for timestep 0 (a strip of it for the
+    large workloads) against the oracle's, by the workload's tolerance."""
     import oracle
+    a, bs_, gys = res.host
     steps, bb, repeats, sample = w.steps, w.bb, 2, "full workload"
+    b_list, gy_list = bs_, gys
     if w.name.startswith("half_storage"):
         bb, repeats, sample = 1, 1, "1 of the 8 minibatch samples (a shared), fp32"
+        nb, ny = w.dj * w.dk, w.di * w.dk
+        b_list, gy_list = [bs_[0][:nb]], [gys[0][:ny]]
     elif w.name == "square_batched":
         sample = "one fw+bw call, all 16 samples"
     elif w.name in ("dense",):
         repeats = 5
-    rng = np.random.default_rng(0)
     bs = max(w.ba, bb)
-    a = rng.standard_normal(w.di * w.dj * w.ba).astype(np.float32)
-    b = rng.standard_normal(w.dj * w.dk * bb).astype(np.float32)
-    gy = rng.standard_normal(w.di * w.dk * bs).astype(np.float32)
-    ga, gb = np.zeros_like(a), np.zeros_like(b)
+    ga, gb = np.zeros_like(a), np.zeros_like(b_list[0])
     best = float("inf")
     for _ in range(repeats):
         t0 = time.perf_counter()
-        for _ in range(steps):
-            oracle.matmul_fw(a, b, w.di, w.dj, w.dk, w.ba, bb, threads)
-            oracle.matmul_bw(a, b, gy, ga, gb, w.di, w.dj, w.dk, w.ba, bb, threads)
+        for t in range(steps):
+            oracle.matmul_fw(a, b_list[t], w.di, w.dj, w.dk, w.ba, bb, threads)
+            oracle.matmul_bw(a, b_list[t], gy_list[t], ga, gb, w.di, w.dj, w.dk, w.ba, bb, threads)
         best = min(best, time.perf_counter() - t0)
     flops = 3 * 2 * w.di * w.dj * w.dk * bs * steps
     try:
         usable = len(os.sched_getaffinity(0))
     except AttributeError:
         usable = os.cpu_count()
-    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    base = {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "host_cores_online": os.cpu_count(), "host_cores_usable": usable,
-            "sample": "%s, best of %d, %.2f s" % (sample, repeats, best)}
+            "sample": "%s, seeded inputs of the workload, best of %d, %.2f s" % (sample, repeats, best)}
+    # parity of the buffers this run timed
+    if w.ba > 1:       # per-sample products: sample 0
+        na, nb, ny = w.di * w.dj, w.dj * w.dk, w.di * w.dk
+        want = oracle.matmul_fw(a[:na], bs_[0][:nb], w.di, w.dj, w.dk, 1, 1, threads)
+        got = res.y[0].to_vector()[:ny]
+        what = "y of sample 0"
+    else:              # shared a: the first columns of y (all of it when small)
+        cols = min(w.dk * w.bb, 64 if w.di * w.dj >= (1 << 24) else w.dk * w.bb)
+        want = oracle.matmul_fw(a, bs_[0][:w.dj * cols], w.di, w.dj, cols, 1, 1, threads)
+        got = res.y[0].to_vector()[:w.di * cols]
+        what = "y of timestep 0" + ("" if cols == w.dk * w.bb else ", first %d columns" % cols)
+    err = _rel(got, want)
+    parity = {"checked": what, "max_abs_err_over_max_abs_ref": err, "tolerance": w.tolerance, "ok": bool(err <= w.tolerance)}
+    return base, parity
 
 
 def _workload(name):
-    """A workload of the table, or its half-storage entry with bfloat16 storage (same shapes, same
-    inputs; not one of the reference's configurations, reported next to them)."""
+    """A workload of the table; `<name>:<storage>` is the same workload (shapes, seeded inputs) with
+    another storage type, e.g. half_storage:bf16, rnn_gate:f16.  Those are not among the reference's
+    configurations and are reported next to them."""
     if name == "half_storage_bf16":
-        w = copy.copy(WORKLOADS["half_storage"])
-        w.name, w.storage = name, "bf16"
+        name = "half_storage:bf16"
+    if ":" in name:
+        base, storage = name.split(":")
+        w = copy.copy(WORKLOADS[base])
+        w.name, w.storage = name, storage
+        if storage != "f32":
+            w.tolerance = 2e-2
         return w
     return WORKLOADS[name]
 
 
-def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False):
+# Kernel launches per matmul_fw + matmul_bw call pair as the library plans them today (the kernel
+# traces in profiles/): one forward launch and both gradients in one launch for the three
+# per-timestep fp32 workloads, three launches for the batched squares, a transposed copy of `a` plus
+# three products for the 16-bit workload; anything else: three.
+LAUNCHES_PER_CALL_PAIR = {"dense": 2, "rnn_gate": 2, "output_projection": 2, "square_batched": 3,
+                          "half_storage": 4, "half_storage:bf16": 4}
+
+
+def _figures(w, per_step_s):
+    tflops = w.flops_per_step() * w.steps / per_step_s / 1e12
+    gbs = w.bytes_per_step() * w.steps / per_step_s / 1e9
+    f_mfma, f_hbm = tflops / PEAK_TFLOPS[w.storage], gbs / PEAK_HBM_GBS
+    return {"tflops": tflops, "frac_mfma_peak": f_mfma, "gbs": gbs, "frac_hbm_peak": f_hbm,
+            "binding_roofline": "mfma" if f_mfma >= f_hbm else "hbm", "frac_binding_roofline": max(f_mfma, f_hbm)}
+
+
+def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False, sustained=False):
     w = _workload(name)
+    base = name.split(":")[0]
     dev = pa.HIP(0) if w.storage == "f32" else pa.HIP16(0, storage=w.storage)
     dev.set_deterministic(deterministic)
-    dev.set_overlap(not in_order)
+    per_timestep = base in PER_TIMESTEP
+    lanes_for_record = not in_order and not per_timestep
+    dev.set_overlap(lanes_for_record)
     res = Resident(dev, w)
-    host_s, ev_s = time_gpu(dev, res, steps, warmup)
-    front = {}
-    if w.storage == "f32":
-        # The fp32 workloads are timed by a C++ caller as well (primitiv's callers are C++): the same
-        # calls on the same buffers.  That loop is the step of record; the interpreter's loop above is
-        # reported beside it (on the dispatch-bound workloads it adds up to a microsecond per call).
-        front = time_front(dev, res, steps, warmup)
-        front["ms_per_step_python_loop"] = ev_s / steps * 1e3
-        front["ms_per_step_python_loop_host_clock"] = host_s / steps * 1e3
-        ev_s = front["ms_per_step_native_raw"] * 1e-3 * steps
-        host_s = front["ms_per_step_native_raw_host_clock"] * 1e-3 * steps
-        # the same loops with every launch on one stream: what the library's second lane for runs of
-        # independent matmul calls (phip_set_overlap) contributes
-        dev.set_overlap(False)
-        one_stream = time_front(dev, res, steps, warmup)
-        dev.set_overlap(not in_order)
-        front["ms_per_step_in_order"] = one_stream["ms_per_step_native_raw"]
-        front["ms_per_step_front_in_order"] = one_stream["ms_per_step_front"]
-    del res
-    dev.close()
-    per_step = ev_s / steps
-    tflops = w.flops_per_step() * w.steps / per_step / 1e12
-    gbs = w.bytes_per_step() * w.steps / per_step / 1e9
-    f_mfma, f_hbm = tflops / PEAK_TFLOPS[w.storage], gbs / PEAK_HBM_GBS
-    launches = 3 * w.steps
-    out = {
-        "workload": name, "dtype": w.storage, "calls_per_step": w.steps,
-        "ms_per_step": per_step * 1e3, "ms_per_step_host_clock": host_s / steps * 1e3,
-        "us_per_kernel_launch": per_step / launches * 1e6,
-        "tflops": tflops, "frac_mfma_peak": f_mfma, "gbs": gbs, "frac_hbm_peak": f_hbm,
-        "binding_roofline": "mfma" if f_mfma >= f_hbm else "hbm",
-        "frac_binding_roofline": max(f_mfma, f_hbm),
-    }
-    out.update(front)
+    loops = Loops(dev, res)
+    dev.gemm_trace(True)
+    loops.raw(1, 0)
+    kernels = dev.gemm_trace(False)[:8]
+    warm_steps, warm_s = loops.settle(warmup)
+    ms, host_ms = loops.raw(steps, 0)                       # the step of record: a C++ caller's loop
+    out = {"workload": name, "dtype": w.storage, "calls_per_step": w.steps, "steps_timed": steps,
+           "warmup_effective_steps": warm_steps, "warmup_effective_s": warm_s,
+           "ms_per_step": ms, "ms_per_step_host_clock": host_ms,
+           "streams": "one" if not lanes_for_record else "library default (two lanes for runs of independent products)",
+           "gemm_kernels_first_timestep": kernels}
+    launches = LAUNCHES_PER_CALL_PAIR.get(name, 3) * w.steps
+    out["kernel_launches_per_step"] = launches
+    out["us_per_kernel_launch"] = ms * 1e3 / launches
+    out.update(_figures(w, ms * 1e-3))
+    out["ms_per_step_front"], out["ms_per_step_front_host_clock"] = loops.front(steps, 2)
+    out["ms_per_step_python_loop"], out["ms_per_step_python_loop_host_clock"] = time_python_loop(dev, res, steps)
+    if per_timestep or w.flops_per_step() / 3 <= 4e9:
+        # the same loops the other way: both lanes (when the record is in order) or one stream
+        dev.set_overlap(not lanes_for_record)
+        loops.raw(max(2, warmup), 0)
+        other, _ = loops.raw(steps, 0)
+        other_front, _ = loops.front(steps, 2)
+        dev.set_overlap(lanes_for_record)
+        two, one = (other, ms) if not lanes_for_record else (ms, other)
+        two_front, one_front = (other_front, out["ms_per_step_front"]) if not lanes_for_record else (out["ms_per_step_front"], other_front)
+        out["ms_per_step_in_order"], out["ms_per_step_front_in_order"] = one, one_front
+        out["frac_binding_roofline_in_order"] = _figures(w, one * 1e-3)["frac_binding_roofline"]
+        if w.storage == "f32":      # 16-bit products always run in order
+            out["ms_per_step_two_lanes"], out["ms_per_step_front_two_lanes"] = two, two_front
+            out["frac_binding_roofline_two_lanes"] = _figures(w, two * 1e-3)["frac_binding_roofline"]
+    if per_timestep and w.storage == "f32" and not deterministic:
+        dev.set_deterministic(True)
+        loops.raw(max(2, warmup), 0)
+        out["ms_per_step_deterministic"], _ = loops.raw(steps, 0)
+        dev.set_deterministic(False)
+    if sustained:
+        n = max(steps, int(SUSTAINED_MIN_SECONDS / (ms * 1e-3)) + 1)
+        s_ms, _ = loops.raw(n, 0)
+        fig = _figures(w, s_ms * 1e-3)
+        out["sustained"] = {"steps": n, "seconds": s_ms * 1e-3 * n, "ms_per_step": s_ms, "tflops": fig["tflops"],
+                            "frac_mfma_peak": fig["frac_mfma_peak"]}
     # HBM traffic per step by the counters (profiles/), next to the algorithmic bytes above
     if name in COUNTER_TRAFFIC_BYTES_PER_STEP:
         traffic = COUNTER_TRAFFIC_BYTES_PER_STEP[name]
         out["counter_traffic_bytes_per_step"] = traffic
-        out["counter_gbs"] = traffic / per_step / 1e9
-        out["counter_frac_hbm_peak"] = traffic / per_step / 1e9 / PEAK_HBM_GBS
+        out["counter_gbs"] = traffic / (ms * 1e-3) / 1e9
+        out["counter_frac_hbm_peak"] = traffic / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS
     if not skip_cpu:
-        out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"], out["parity_in_run"] = cpu_baseline(w, res)
+    del loops, res
+    dev.close()
     return out
 
 
@@ -454,14 +542,133 @@ def measure_conv(reps=10):
     return out
 
 
+def _timed_native(fn, steps, warmup):
+    ev, host = ctypes.c_float(), ctypes.c_double()
+    _lib.check(fn(steps, warmup, ctypes.byref(ev), ctypes.byref(host)))
+    return ev.value / steps, host.value / steps
+
+
+# Device calls of one LSTM timestep as primitiv's graph issues them (bench_native.cc: phip_bench_lstm_loop).
+LSTM_CALLS_FORWARD = 17      # 2 strided copies (concat), matmul, bias add, 4 slices, 4 activations, 5 elementwise
+LSTM_CALLS_BACKWARD = 40     # 17 zero fills, 10 elementwise gradients, 4 + 2 strided copies, matmul_bw, 3 in-place adds ... per timestep
+
+
+def measure_lstm(storage, steps, warmup, hidden=650, batch=64, timesteps=35):
+    """One LSTM layer of the reference's language model (examples/ptb/ptb_rnnlm_lstm.cc:69-112:
+    W {4*hidden, 2*hidden}, minibatch 64, 35 timesteps unrolled), forward through the timesteps and
+    backward through time, every device call as primitiv's Graph would make it (zero-filled gradients
+    included).  A step is the whole sequence; reported per timestep, in order and with the library's
+    default (which engages its second lane only in runs of matmul calls, so here it should not differ)."""
+    from primitiv_amd.configs import Randomizer
+    S = pa.Shape
+    dev = pa.HIP(0) if storage == "f32" else pa.HIP16(0, storage=storage)
+    rng = Randomizer(0)
+    H, I, B, T = hidden, hidden, batch, timesteps
+    W = dev.new_tensor_by_vector(S([4 * H, I + H]), rng.uniform(-0.1, 0.1, 4 * H * (I + H)))
+    b = dev.new_tensor_by_vector(S([4 * H]), rng.uniform(-0.1, 0.1, 4 * H))
+    xs = [dev.new_tensor_by_vector(S([I], B), rng.uniform(-0.1, 0.1, I * B)) for _ in range(T)]
+    gys = [dev.new_tensor_by_vector(S([H], B), rng.normal(0.0, 1e-2, H * B)) for _ in range(T)]
+    gW = dev.new_tensor_by_constant(W.shape(), 0)
+    gb = dev.new_tensor_by_constant(b.shape(), 0)
+    arr = lambda ts: (ctypes.c_void_p * T)(*[t.handle() for t in ts])
+    px, pgy = arr(xs), arr(gys)
+    d = _LstmDims(I, H, B, T)
+    L, code = _native(), STORAGE_CODE[storage]
+
+    def loop(forward_only):
+        return lambda n, wu, ev, host: L.phip_bench_lstm_loop(dev.ctx(), code, ctypes.byref(d), W.handle(), b.handle(),
+                                                              gW.handle(), gb.handle(), px, pgy, None, None,
+                                                              int(forward_only), n, wu, ev, host)
+
+    out = {"layer": "LSTM %d -> %d, minibatch %d, %d timesteps, W {%d,%d}" % (I, H, B, T, 4 * H, I + H), "dtype": storage,
+           "device_calls_per_timestep": {"forward": LSTM_CALLS_FORWARD, "backward": LSTM_CALLS_BACKWARD},
+           "steps_timed": steps}
+    for key, overlap in (("in_order", False), ("library_default", True)):
+        dev.set_overlap(overlap)
+        _timed_native(loop(False), max(2, warmup), 0)
+        fw_ms, fw_host = _timed_native(loop(True), steps, 1)
+        all_ms, all_host = _timed_native(loop(False), steps, 1)
+        out[key] = {"us_per_timestep_forward": fw_ms * 1e3 / T, "us_per_timestep_forward_backward": all_ms * 1e3 / T,
+                    "us_per_timestep_forward_backward_host_clock": all_host * 1e3 / T,
+                    "us_per_timestep_forward_host_clock": fw_host * 1e3 / T}
+    flops = 3 * 2 * (4 * H) * (I + H) * B
+    t = out["in_order"]["us_per_timestep_forward_backward"] * 1e-6
+    out["matmul_tflops_of_the_timestep"] = flops / t / 1e12
+    out["us_per_device_call"] = out["in_order"]["us_per_timestep_forward_backward"] / (LSTM_CALLS_FORWARD + LSTM_CALLS_BACKWARD)
+    dev.gemm_trace(True)
+    _timed_native(loop(False), 1, 0)
+    names = dev.gemm_trace(False)
+    out["gemm_kernels"] = sorted(set(names))
+    del W, b, xs, gys, gW, gb
+    dev.close()
+    return out
+
+
+SWEEP_SQUARES = [256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096]
+# layers of the reference's examples: (name, di, dj, minibatch)
+SWEEP_LAYERS = [
+    ("mnist_hidden", 800, 784, 200),        # examples/mnist/mnist.cc:58-80
+    ("mnist_output", 10, 800, 200),
+    ("ptb_lstm_b20", 2600, 1300, 20),       # examples/ptb/ptb_rnnlm_lstm.cc:86-101, minibatch 20
+    ("ptb_lstm_b64", 2600, 1300, 64),
+    ("ptb_projection_b20", 10000, 650, 20),  # :125
+]
+
+
+def measure_sweep(reps=20):
+    """Shape sweep, every launch on one stream: unbatched squares M = N = K and the reference examples' layers
+    (a shared, minibatch folded into columns), forward and backward timed apart, fp32 and fp16 storage, with
+    the kernels each went to.  Neighbouring squares whose efficiency differs by more than 1.5x are flagged."""
+    from primitiv_amd.configs import Workload
+    rows = []
+    for storage in ("f32", "f16"):
+        dev = pa.HIP(0) if storage == "f32" else pa.HIP16(0, storage=storage)
+        dev.set_overlap(False)
+        cases = [("square_%d" % n, n, n, n, 1, 1) for n in SWEEP_SQUARES]
+        cases += [(name, di, dj, 1, 1, bs) for name, di, dj, bs in SWEEP_LAYERS]
+        prev = None
+        for name, di, dj, dk, ba, bb in cases:
+            dist = ("normal", 0.0, 1.0)
+            w = Workload(name, di, dj, dk, ba, bb, 1, ("uniform", -0.1, 0.1), dist, dist, storage=storage)
+            res = Resident(dev, w)
+            loops = Loops(dev, res)
+            row = {"shape": name, "dtype": storage, "di": di, "dj": dj, "dk": dk * bb}
+            third = w.flops_per_step() / 3
+            for which, key, flops in ((1, "fw", third), (2, "bw", 2 * third)):
+                dev.gemm_trace(True)
+                loops.raw(1, 0, which)
+                row[key + "_kernels"] = "+".join(dev.gemm_trace(False))
+                n = max(3, min(reps, int(0.05 / max(1e-6, flops / 50e12))))
+                loops.raw(n, 0, which)
+                ms, _ = loops.raw(n, 0, which)
+                row[key + "_us"] = ms * 1e3
+                row[key + "_tflops"] = flops / (ms * 1e-3) / 1e12
+                row[key + "_frac_mfma_peak"] = row[key + "_tflops"] / PEAK_TFLOPS[storage]
+            if name.startswith("square") and prev is not None:
+                for key in ("fw", "bw"):
+                    r = row[key + "_frac_mfma_peak"] / prev[key + "_frac_mfma_peak"]
+                    if r > 1.5 or r < 1 / 1.5:
+                        row.setdefault("cliff", []).append("%s x%.2f vs %s" % (key, r, prev["shape"]))
+            prev = row if name.startswith("square") else None
+            rows.append(row)
+            print("# %-20s %s  fw %8.1f us %7.1f TF (%4.1f%%) %-22s  bw %8.1f us %7.1f TF (%4.1f%%) %-30s %s"
+                  % (name, storage, row["fw_us"], row["fw_tflops"], 100 * row["fw_frac_mfma_peak"], row["fw_kernels"],
+                     row["bw_us"], row["bw_tflops"], 100 * row["bw_frac_mfma_peak"], row["bw_kernels"],
+                     " ".join(row.get("cliff", []))), file=sys.stderr, flush=True)
+            del loops, res
+        dev.close()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
-                    help="all or one of: " + ", ".join(list(WORKLOADS) + ["half_storage_bf16"]))
-    ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle")
+                    help="all or one of: " + ", ".join(list(WORKLOADS)) + "; name:storage runs a workload with "
+                         "another storage type (half_storage:bf16, rnn_gate:f16, ...)")
+    ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU oracle (nor check against it)")
     ap.add_argument("--in-order", action="store_true",
                     help="every launch on one stream (phip_set_overlap off): per-kernel durations under a profiler")
     ap.add_argument("--deterministic", action="store_true",
@@ -473,6 +680,11 @@ def main():
                     help="measure the elementwise kernels' streaming rates instead of the matmul workloads")
     ap.add_argument("--conv", action="store_true",
                     help="measure conv2d and max_pool2d on image-model layer shapes instead of the matmul workloads")
+    ap.add_argument("--lstm", action="store_true",
+                    help="one LSTM layer of the reference's language model, forward and backward through time, "
+                         "device call by device call")
+    ap.add_argument("--sweep", action="store_true",
+                    help="shape sweep (unbatched squares, the reference examples' layers), fp32 and fp16, with kernel names")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path "
@@ -487,6 +699,23 @@ def main():
                           "data": "synthetic", "kernels": measure_conv()}))
         return
 
+    if args.lstm:
+        layers = [measure_lstm(st, max(2, min(args.steps, 10)), args.warmup) for st in ("f32", "f16", "bf16")]
+        for l in layers:
+            print("# lstm %s: %.1f us / timestep forward + backward in order (%.1f forward), %.1f library default; "
+                  "%.2f us per device call" % (l["dtype"], l["in_order"]["us_per_timestep_forward_backward"],
+                                                l["in_order"]["us_per_timestep_forward"],
+                                                l["library_default"]["us_per_timestep_forward_backward"],
+                                                l["us_per_device_call"]), file=sys.stderr, flush=True)
+        print(json.dumps({"metric": "LSTM layer, microseconds per timestep (forward + backward through time)",
+                          "unit": "us", "n_gpus": 1, "data": "synthetic", "higher_is_better": False, "layers": layers}))
+        return
+
+    if args.sweep:
+        print(json.dumps({"metric": "matmul shape sweep, TFLOP/s and fraction of the MFMA peak", "n_gpus": 1,
+                          "data": "synthetic", "peaks_tflops": PEAK_TFLOPS, "rows": measure_sweep()}))
+        return
+
     if args.traffic_calibration:
         dev = pa.HIP(0)
         n = 64 << 20
@@ -496,48 +725,53 @@ def main():
         del x, y
         dev.close()
 
-    names = list(WORKLOADS) + ["half_storage_bf16"] if args.workload == "all" else [args.workload]
-    if HEADLINE not in names and args.workload == "all":
-        names.append(HEADLINE)
+    # the reference's five configurations, then the same shapes with other storage types (reported extras)
+    extras = ["half_storage:bf16", "rnn_gate:f16", "rnn_gate:bf16", "output_projection:f16", "output_projection:bf16"]
+    names = list(WORKLOADS) + extras if args.workload == "all" else [args.workload]
     results = {}
     for n in names:
         steps = args.steps if not n.startswith("half_storage") else max(1, min(args.steps, 5))
-        # the CPU figure of the bf16 variant would repeat the fp16 one: same shapes, fp32 on the CPU
-        results[n] = measure(n, steps, args.warmup, args.skip_cpu or n == "half_storage_bf16", args.deterministic, args.in_order)
-        print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)%s"
-              % (n, results[n]["ms_per_step"], results[n]["tflops"], 100 * results[n]["frac_mfma_peak"],
-                 results[n]["gbs"], 100 * results[n]["frac_hbm_peak"],
-                 "  [%.3f ms/step with every launch on one stream]" % results[n]["ms_per_step_in_order"]
-                 if "ms_per_step_in_order" in results[n] else ""), file=sys.stderr, flush=True)
+        # the CPU figure of a storage variant would repeat its fp32 / fp16 one: same shapes, fp32 on the CPU
+        base = n.split(":")[0]
+        results[n] = measure(n, steps, args.warmup, args.skip_cpu or (":" in n and base != "half_storage"),
+                             args.deterministic, args.in_order, sustained=base in (HEADLINE, "half_storage"))
+        r = results[n]
+        print("# %s: %.3f ms/step  %.2f TFLOP/s (%.1f%% of MFMA peak)  %.0f GB/s (%.1f%% of HBM peak)  [%s]%s%s"
+              % (n, r["ms_per_step"], r["tflops"], 100 * r["frac_mfma_peak"], r["gbs"], 100 * r["frac_hbm_peak"],
+                 "+".join(r["gemm_kernels_first_timestep"]),
+                 "  [%.3f ms/step on two lanes]" % r["ms_per_step_two_lanes"] if "ms_per_step_two_lanes" in r else "",
+                 "  [sustained %.1f s: %.2f TFLOP/s]" % (r["sustained"]["seconds"], r["sustained"]["tflops"])
+                 if "sustained" in r else ""), file=sys.stderr, flush=True)
 
     head = results.get(HEADLINE) or results[names[0]]
-    w = WORKLOADS[head["workload"]]
+    w = _workload(head["workload"])
     # Dominant kernel of the headline workload: the 128x128x32 fp32 MFMA GEMM
     # with global-to-LDS loads (three operand-layout instantiations, one launch
     # each per step, equal flops); its average launch duration is the event
     # time over the launches.
-    launch_s = head["ms_per_step"] * 1e-3 / (3 * w.steps)
-    flops_per_launch = w.flops_per_step() / 3
+    launch_s = head["ms_per_step"] * 1e-3 / head["kernel_launches_per_step"]
+    flops_per_launch = w.flops_per_step() * w.steps / head["kernel_launches_per_step"]
     roofline = {
         "bound": "mfma", "achieved": flops_per_launch / launch_s / 1e12, "peak": PEAK_TFLOPS[w.storage],
         "unit": "TFLOP/s", "frac": flops_per_launch / launch_s / 1e12 / PEAK_TFLOPS[w.storage],
         "traffic": HEADLINE_TRAFFIC_BYTES if head["workload"] == HEADLINE else None,
-        "kernel": "gemm_f32_lds_kernel<A_KMAJOR,B_KMAJOR,false> (fw, ga, gb)",
+        "kernel": "gemm_f32_lds_kernel<A_KMAJOR,B_KMAJOR,false> (fw, ga, gb)" if head["workload"] == HEADLINE
+                  else "+".join(head["gemm_kernels_first_timestep"]),
         "flops_per_launch": flops_per_launch, "avg_launch_ms": launch_s * 1e3,
     }
     line = {
         "metric": "matmul fw+bw TFLOP/s", "value": head["tflops"], "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": head["steps_timed"], "warmup": args.warmup,
+        "warmup_effective_steps": head["warmup_effective_steps"], "warmup_effective_s": head["warmup_effective_s"],
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32" if w.storage == "f32" else w.storage, "data": "synthetic",
-        "config": {"workload": "%s: a,b,gy {%d,%d}x%d fp32, fw + both gradients"
-                   % (head["workload"], w.di, w.dj, w.bs),
-                   "streams": "one (--in-order)" if args.in_order else
-                              "library default: a second stream for runs of independent matmul calls of at most 4 GFLOP (%s)"
-                              % ("this workload's products are larger and run in order" if w.flops_per_step() / 3 > 4e9
-                                 else "this workload's calls use it"),
+        "vs_baseline": None, "dtype": w.storage, "data": "synthetic",
+        "config": {"workload": "%s: a,b,gy {%d,%d}x%d %s, fw + both gradients"
+                   % (head["workload"], w.di, w.dj, w.bs, w.storage),
+                   "streams": head["streams"],
                    "tolerance": "max|x-ref|/max|ref| <= %.0e vs CPU oracle" % w.tolerance},
         "frac_of_mfma_peak": head["frac_mfma_peak"],
+        "sustained": head.get("sustained"),
+        "parity_in_run": head.get("parity_in_run"),
         "roofline": roofline,
         "cpu_baseline": head.get("cpu_baseline"),
         "workloads": results,

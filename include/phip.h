@@ -241,6 +241,16 @@ int phip_matmul_bw_bf16(phip_ctx *ctx, const void *a, const void *b, const void 
                         void *ga, void *gb,
                         uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb);
 
+/* Which kernels the matrix products went to.  No counterpart in the reference
+ * (its devices hand every product to a vendor GEMM).  Copies the names of the
+ * GEMM kernels launched by this context's matmul and convolution calls since
+ * the previous call into buf (space-separated, in launch order per stream;
+ * truncated to buf_size; buf may be NULL), forgets them, and switches the
+ * note-taking on (on != 0) or off (the default).  For benchmarks and tests
+ * that report or assert the kernel family a shape is served by; costs nothing
+ * while off. */
+int phip_gemm_trace(phip_ctx *ctx, int on, char *buf, size_t buf_size);
+
 /* ---- elementwise operations around the matmul ------------------------------
  * The layers of every primitiv example wrap the matmul in a bias add and an
  * activation (examples/mnist/mnist.cc:74,80; examples/ptb/ptb_rnnlm_lstm.cc:

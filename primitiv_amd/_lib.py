@@ -180,6 +180,7 @@ SIGNATURES = {
     "phip_random_log_normal_bf16": [_vp, _u64, _u64, _f, _f, _vp, _sz],
     "phip_matmul_fw_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_f32_noalloc": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
+    "phip_gemm_trace": [_vp, ctypes.c_int, ctypes.c_char_p, _sz],
     "phip_matmul_fw_f16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_bf16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_bw_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],

@@ -10,8 +10,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libphip.so")
-# host-only timing loops for bench.py, linked against libphip
-BENCH_LIB_PATH = os.path.join(HERE, "libphip_bench.so")
 
 SOURCES = [
     "phip_runtime.hip",
@@ -60,9 +58,6 @@ def build(jobs=4, verbose=True):
         objs = list(ex.map(_compile, SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     subprocess.check_call(cmd)
-    subprocess.check_call(["g++", "-O2", "-std=c++11", "-fPIC", "-shared", "-Wall", "-Wextra",
-                           os.path.join(HERE, "bench_front.cc"), "-o", BENCH_LIB_PATH,
-                           "-L" + HERE, "-lphip", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB_PATH)
     return LIB_PATH

@@ -65,9 +65,15 @@ int gemm_f32(phip_ctx *ctx, const Gemm &p) {
   StagedPlan plan;
   plan_staged(ctx, p, &plan);
   switch (plan.shape) {
-    case StagedShape::k128x128x16: return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, plan);
-    case StagedShape::k64x64x32: return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, plan);
-    default: return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, plan);
+    case StagedShape::k128x128x16:
+      note_kernel(ctx, "f32_staged128");
+      return launch_tile<128, 128, 16, 2, 2, 1, 4>(ctx, p, plan);
+    case StagedShape::k64x64x32:
+      note_kernel(ctx, "f32_staged64");
+      return launch_tile<64, 64, 32, 2, 2, 1, 2>(ctx, p, plan);
+    default:
+      note_kernel(ctx, "f32_staged32");
+      return launch_tile<32, 32, 64, 1, 1, 4, 2>(ctx, p, plan);
   }
 }
 

@@ -54,6 +54,7 @@ int gemm_f32_direct(phip_ctx *ctx, const Gemm &p, bool *handled) {
   *handled = false;
   DirectPlan plan;
   if (!plan_direct(ctx, p, &plan)) return PHIP_OK;
+  note_kernel(ctx, "f32_direct");
   *handled = true;
   if (plan.waves == 8) {
     if (plan.tn == 2) return launch_direct<1, 2, 8, 8>(ctx, p, plan);

@@ -415,6 +415,7 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
 #undef PHIP_LDS64
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, side == LBM ? (splits > 1 ? "f32_lds128_split" : "f32_lds128") : (splits > 1 ? "f32_lds64_split" : "f32_lds64"));
   *handled = true;
   return PHIP_OK;
 }

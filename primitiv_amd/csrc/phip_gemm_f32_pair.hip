@@ -83,6 +83,7 @@ int gemm_f32_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, bool *ha
   }
   const long padded = (p1.grid + 7) / 8 * 8;
   if (padded + p2.grid > 0x7fffffffL) return PHIP_OK;
+  note_kernel(ctx, "f32_pair");
   *handled = true;
 #define PHIP_PAIR(FIRST, U2)                                                                                  \
   hipLaunchKernelGGL((gemm_f32_pair_kernel<FIRST, U2>), dim3((unsigned)(padded + p2.grid)), dim3(kThreads), 0, \

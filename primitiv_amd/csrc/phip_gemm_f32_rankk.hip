@@ -29,6 +29,7 @@ int gemm_f32_rankk(phip_ctx *ctx, const Gemm &p, bool *handled) {
   if (rc != PHIP_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)plan.tiles), dim3(kThreads), kRankLdsBytes, ctx->stream, plan.d);
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, "f32_rankk");
   *handled = true;
   return PHIP_OK;
 }

@@ -43,6 +43,7 @@ int gemm_f32_slab(phip_ctx *ctx, const Gemm &p, bool *handled) {
   else PHIP_SLAB_G(kSlotGemmF32Slab + 2, true, true);
 #undef PHIP_SLAB_G
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, "f32_slab");
   *handled = true;
   return PHIP_OK;
 }

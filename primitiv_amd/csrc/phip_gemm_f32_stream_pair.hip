@@ -79,6 +79,7 @@ int gemm_f32_stream_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, b
   hipLaunchKernelGGL(kern, dim3((unsigned)(s.padded + sp.grid)), dim3(kThreads), kStreamPairLdsBytes, ctx->stream,
                      rp.d, sp.d, s);
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, "f32_stream_pair");
   *handled = true;
   return PHIP_OK;
 }

@@ -121,6 +121,7 @@ int gemm_f32_tile16(phip_ctx *ctx, const Gemm &p, bool *handled) {
     hipLaunchKernelGGL(gemm_f32_tile16_kernel<false>, dim3((unsigned)tiles16), dim3(kT16Threads), 0, ctx->stream, d);
   }
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, "f32_tile16");
   *handled = true;
   return PHIP_OK;
 }

@@ -468,8 +468,15 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
   auto tiles = [&](int bm, int bn) {
     return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch;
   };
-  if (tiles(128, 128) >= cus) return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
-  if (tiles(64, 64) >= cus) return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
+  if (tiles(128, 128) >= cus) {
+    note_kernel(ctx, "h16_staged128");
+    return launch_tile_h<128, 128, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
+  }
+  if (tiles(64, 64) >= cus) {
+    note_kernel(ctx, "h16_staged64");
+    return launch_tile_h<64, 64, 32, 2, 2, 1, BF16>(ctx, p, a, vec_a, vec_b);
+  }
+  note_kernel(ctx, "h16_staged32");
   return launch_tile_h<32, 32, 64, 1, 1, 4, BF16>(ctx, p, a, vec_a, vec_b, true);
 }
 

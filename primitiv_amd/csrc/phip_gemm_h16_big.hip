@@ -675,6 +675,7 @@ int gemm_h16_big(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   a.accumulate = p.accumulate ? 1 : 0;
   a.a_bytes = (uint32_t)a_bytes;
   a.b_bytes = (uint32_t)b_bytes;
+  note_kernel(ctx, side == kTile<4> ? "h16_lds256" : "h16_lds128");
   *handled = true;
   if (side == kTile<4>) return elem == Elem::BF16 ? launch_big<true, 4>(ctx, p, a) : launch_big<false, 4>(ctx, p, a);
   return elem == Elem::BF16 ? launch_big<true, 2>(ctx, p, a) : launch_big<false, 2>(ctx, p, a);

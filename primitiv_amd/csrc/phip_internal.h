@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -81,6 +82,10 @@ struct phip_ctx {
   bool fixed_mode = false;
   // The second lane for matrix products; null in the side lane's own context.
   phip::Lanes *lanes = nullptr;
+  // Names of the matrix-product kernels launched on this context since the last phip_gemm_trace call,
+  // kept only while tracing is switched on (benchmarks and tests ask which kernel a shape went to).
+  bool trace_on = false;
+  std::string trace;
 };
 
 struct phip_event {
@@ -152,6 +157,13 @@ int lanes_wait_host(phip_ctx *ctx);
 // What is enqueued on the main lane next comes after the side lane's work, and touches no tensor (an event).
 int lanes_order_main_after_side(phip_ctx *ctx);
 int lanes_place(phip_ctx *ctx, const MemRange *ranges, int n, bool may_overlap, phip_ctx **run_on);
+
+// Notes that a matrix product went to the kernel `name` (phip_gemm_trace).
+inline void note_kernel(phip_ctx *ctx, const char *name) {
+  if (!ctx->trace_on || ctx->trace.size() > 4000) return;
+  if (!ctx->trace.empty()) ctx->trace += ' ';
+  ctx->trace += name;
+}
 
 // Entries of phip_ctx::tile_tickets.
 constexpr int kTicketSlots = 65536;

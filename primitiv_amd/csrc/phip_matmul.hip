@@ -220,6 +220,23 @@ int phip_matmul_fw_f32_noalloc(phip_ctx *ctx, const float *a, const float *b, fl
   return matmul_fw(ctx, Elem::F32, a, b, y, di, dj, dk, ba, bb);
 }
 
+int phip_gemm_trace(phip_ctx *ctx, int on, char *buf, size_t buf_size) {
+  PHIP_REQUIRE(ctx != nullptr, "null context");
+  phip_ctx *side = ctx->lanes != nullptr ? ctx->lanes->side : nullptr;
+  if (buf != nullptr && buf_size > 0) {
+    std::string all = ctx->trace;
+    if (side != nullptr && !side->trace.empty()) all += (all.empty() ? "" : " ") + side->trace;
+    std::snprintf(buf, buf_size, "%s", all.c_str());
+  }
+  ctx->trace.clear();
+  ctx->trace_on = on != 0;
+  if (side != nullptr) {
+    side->trace.clear();
+    side->trace_on = on != 0;
+  }
+  return PHIP_OK;
+}
+
 int phip_matmul_bw_f32(phip_ctx *ctx, const float *a, const float *b, const float *gy, float *ga,
                        float *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
   return matmul_bw(ctx, Elem::F32, a, b, gy, ga, gb, di, dj, dk, ba, bb);

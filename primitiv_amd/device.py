@@ -421,6 +421,13 @@ class HIP:
         default); off: every launch on one stream."""
         _lib.call("phip_set_overlap", self._ctx, 1 if on else 0)
 
+    def gemm_trace(self, on=True):
+        """Names of the GEMM kernels that this device's matmul calls went to since the previous call
+        (a list, launch order per stream); `on` switches the note-taking on or off from here on."""
+        buf = ctypes.create_string_buffer(4096)
+        _lib.call("phip_gemm_trace", self._ctx, 1 if on else 0, buf, len(buf))
+        return buf.value.decode().split()
+
     # -- storage ----------------------------------------------------------
     def _elements_to_bytes(self, n):
         return self._ITEMSIZE * n
