@@ -683,6 +683,7 @@ def main():
     ap.add_argument("--lstm", action="store_true",
                     help="one LSTM layer of the reference's language model, forward and backward through time, "
                          "device call by device call")
+    ap.add_argument("--storage", default="all", help="with --lstm: f32, f16, bf16 or all")
     ap.add_argument("--sweep", action="store_true",
                     help="shape sweep (unbatched squares, the reference examples' layers), fp32 and fp16, with kernel names")
     args = ap.parse_args()
@@ -700,7 +701,7 @@ def main():
         return
 
     if args.lstm:
-        layers = [measure_lstm(st, max(2, min(args.steps, 10)), args.warmup) for st in ("f32", "f16", "bf16")]
+        layers = [measure_lstm(st, max(2, min(args.steps, 10)), args.warmup) for st in (("f32", "f16", "bf16") if args.storage == "all" else (args.storage,))]
         for l in layers:
             print("# lstm %s: %.1f us / timestep forward + backward in order (%.1f forward), %.1f library default; "
                   "%.2f us per device call" % (l["dtype"], l["in_order"]["us_per_timestep_forward_backward"],

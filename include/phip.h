@@ -114,6 +114,24 @@ int phip_set_deterministic(phip_ctx *ctx, int on);
  * default of contexts created afterwards.  The call itself waits for neither
  * lane on the host. */
 int phip_set_overlap(phip_ctx *ctx, int on);
+/* Zero fills that are only noted.  No counterpart in the reference's interface.
+ * primitiv's backward pass gives every gradient a zero-filled tensor and then
+ * calls an operator that adds into it (primitiv/core/graph.cc:192-216) - two
+ * launches per gradient where the tensors are small and a launch costs more
+ * than its work.  By default phip_fill_* with the value +0 launches nothing:
+ * the range is noted, and the next entry point of the context either is a
+ * gradient operation (phip_unary_bw_*, phip_const_bw_*, phip_pown_bw_*,
+ * phip_binary_bw_*, phip_inplace_add_*, phip_inplace_subtract_*) whose output
+ * is exactly that range - it then writes 0 + value instead of reading and
+ * adding, the same bits - or launches the noted fills first, in the order they
+ * were asked for.  Nothing the caller can observe changes: every entry point
+ * that reads, writes, copies or waits sees the memory as if the fill had run
+ * when it was called, and a block handed back with phip_pool_free simply
+ * forgets its fill.  Memory that the caller touches behind the library's back
+ * (its own HIP calls on the raw pointers) would see the difference; on == 0
+ * launches every fill at once, as does the environment variable
+ * PHIP_DEFER_ZERO_FILLS=0 for contexts created afterwards. */
+int phip_set_deferred_zero_fill(phip_ctx *ctx, int on);
 
 /* ---- raw memory -----------------------------------------------------------
  * Reference: the allocator / deleter lambdas handed to MemoryPool

@@ -181,6 +181,7 @@ SIGNATURES = {
     "phip_matmul_fw_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_f32_noalloc": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_gemm_trace": [_vp, ctypes.c_int, ctypes.c_char_p, _sz],
+    "phip_set_deferred_zero_fill": [_vp, ctypes.c_int],
     "phip_matmul_fw_f16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_fw_bf16": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "phip_matmul_bw_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -35,6 +36,18 @@ struct MemRange {
   uintptr_t lo, hi;
   bool write;
 };
+// A zero fill that has been asked for and not launched (phip_elementwise.hip): primitiv's backward
+// pass gives every gradient a zero-filled tensor and then lets an operator add into it, which for
+// the small per-timestep tensors of a recurrent network is two launches where one that writes
+// instead of adding does the same.  A zero fill is only noted; the next entry point either takes
+// the note for an output that it would add into (and overwrites instead: same bits, 0 + v), or
+// launches the fill first.  Notes never outlive the next entry point that enqueues work.
+struct PendingZero {
+  uintptr_t lo;
+  size_t bytes;
+  int elem;  // 0: float, 1: f16, 2: bf16 (which fill kernel to launch)
+};
+
 struct Lanes {
   phip_ctx *side = nullptr;
   bool enabled = true;
@@ -86,6 +99,12 @@ struct phip_ctx {
   // kept only while tracing is switched on (benchmarks and tests ask which kernel a shape went to).
   bool trace_on = false;
   std::string trace;
+  // Zero fills noted and not yet launched (see phip::PendingZero); `defer_zero_fills` off: every fill launches.
+  // Guarded by `mutex` (a handle deleter on another thread drops the notes of the block it returns);
+  // zeros_count mirrors zeros.size() so that entry points can skip the lock when there is nothing.
+  std::vector<phip::PendingZero> zeros;
+  std::atomic<int> zeros_count{0};
+  bool defer_zero_fills = true;
 };
 
 struct phip_event {
@@ -116,10 +135,31 @@ struct phip_event {
   PHIP_REQUIRE((ctx) != nullptr, "null context");                             \
   PHIP_HIP(hipSetDevice((ctx)->device))
 
-// The same for every entry point that enqueues work on the context's stream or waits for it: the
-// stream first waits for the matrix products that run on the side lane.
+// Launches the zero fills that were noted and not taken (no-op when there are none).
+#define PHIP_FLUSH_ZEROS(ctx)                                                 \
+  do {                                                                        \
+    if ((ctx)->zeros_count.load(std::memory_order_relaxed) != 0) {            \
+      const int phip_zero_rc__ = phip::zeros_flush(ctx);                      \
+      if (phip_zero_rc__ != PHIP_OK) return phip_zero_rc__;                   \
+    }                                                                         \
+  } while (0)
+
+// For the entry points that may take a noted zero fill for an output they add into: as PHIP_ENTER
+// but the notes stay; the entry point calls zeros_take for such outputs and then PHIP_FLUSH_ZEROS.
+#define PHIP_ENTER_KEEP_ZEROS(ctx)                                            \
+  PHIP_ENTER_HOST(ctx);                                                       \
+  do {                                                                        \
+    if ((ctx)->lanes != nullptr) {                                            \
+      const int phip_join_rc__ = phip::lanes_join(ctx);                       \
+      if (phip_join_rc__ != PHIP_OK) return phip_join_rc__;                   \
+    }                                                                         \
+  } while (0)
+
+// The same for every entry point that enqueues work on the context's stream or waits for it: noted
+// zero fills are launched, then the stream waits for the matrix products that run on the side lane.
 #define PHIP_ENTER(ctx)                                                       \
   PHIP_ENTER_HOST(ctx);                                                       \
+  PHIP_FLUSH_ZEROS(ctx);                                                      \
   do {                                                                        \
     if ((ctx)->lanes != nullptr) {                                            \
       const int phip_join_rc__ = phip::lanes_join(ctx);                       \
@@ -132,6 +172,7 @@ struct phip_event {
 // for the other and leaves the lanes as they are.
 #define PHIP_ENTER_BLOCKING(ctx)                                              \
   PHIP_ENTER_HOST(ctx);                                                       \
+  PHIP_FLUSH_ZEROS(ctx);                                                      \
   do {                                                                        \
     if ((ctx)->lanes != nullptr) {                                            \
       const int phip_join_rc__ = phip::lanes_wait_host(ctx);                  \
@@ -143,6 +184,20 @@ struct phip_event {
 #define PHIP_LAUNCH_CHECK() PHIP_HIP(hipGetLastError())
 
 namespace phip {
+
+// Noted zero fills (phip_elementwise.hip).  zeros_flush launches them all, in the order they were
+// asked for.  zeros_take: true when exactly [p, p + bytes) is noted as zero; the note is removed and
+// the caller writes the range instead of adding into it.  zeros_drop forgets the notes inside a range
+// whose contents no longer matter (a block handed back to the pool).
+int zeros_flush(phip_ctx *ctx);
+bool zeros_take(phip_ctx *ctx, const void *p, size_t bytes);
+// True when [p, p + bytes) and [q, q + qbytes) share memory (q may be null).  An output that is also
+// read as an operand must see its fill before the operation, so its note is not taken.
+inline bool shares_memory(const void *p, size_t bytes, const void *q, size_t qbytes) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(q);
+  return q != nullptr && a < b + qbytes && b < a + bytes;
+}
+void zeros_drop(phip_ctx *ctx, const void *p, size_t bytes);
 
 // phip_lanes.hip.  lanes_join: the main lane waits for everything on the side lane (no-op when
 // nothing is in flight there).  lanes_place: picks the lane of a matrix product with the given

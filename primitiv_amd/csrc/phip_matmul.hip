@@ -55,6 +55,7 @@ static int place(phip_ctx *ctx, Elem elem, const MemRange *ranges, int n, uint32
 static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, void *y, uint32_t di,
                      uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
   PHIP_ENTER_HOST(ctx);
+  PHIP_FLUSH_ZEROS(ctx);
   int rc = check_matmul_args(a, b, y, di, dj, dk, ba, bb);
   if (rc != PHIP_OK) return rc;
   {
@@ -112,6 +113,7 @@ static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, voi
 static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, const void *gy, void *ga,
                      void *gb, uint32_t di, uint32_t dj, uint32_t dk, uint32_t ba, uint32_t bb) {
   PHIP_ENTER_HOST(ctx);
+  PHIP_FLUSH_ZEROS(ctx);
   int rc = check_matmul_args(a, b, gy, di, dj, dk, ba, bb);
   if (rc != PHIP_OK) return rc;
   PHIP_REQUIRE(ga != nullptr && gb != nullptr, "null gradient pointer");

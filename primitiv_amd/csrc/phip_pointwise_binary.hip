@@ -123,10 +123,12 @@ __global__ __launch_bounds__(kBlock) void scalar_fw_kernel(const T *x, const T *
 // ---- backward, same batch on both sides ---------------------------------------
 
 // ga[i] += da, gb[i] += db.  `same` is set when ga and gb are one array (both
-// operands are the same tensor): then the array receives da + db.
+// operands are the same tensor): then the array receives da + db.  acc_a / acc_b off: that
+// gradient's old value counts as zero and is not read.
 template <typename T, typename OP, bool VEC>
 __global__ __launch_bounds__(kBlock) void binary_bw_flat_kernel(const T *a, const T *b, const T *y, const T *gy,
-                                                                 T *ga, T *gb, size_t n, bool same) {
+                                                                 T *ga, T *gb, size_t n, bool same, bool acc_a,
+                                                                 bool acc_b) {
   const size_t stride = (size_t)gridDim.x * kBlock;
   const size_t first = (size_t)blockIdx.x * kBlock + threadIdx.x;
   auto one = [&](size_t i) {
@@ -134,10 +136,10 @@ __global__ __launch_bounds__(kBlock) void binary_bw_flat_kernel(const T *a, cons
     OP::bw(OP::kA ? to_f32(a[i]) : 0.f, OP::kB ? to_f32(b[i]) : 0.f, OP::kY ? to_f32(y[i]) : 0.f, to_f32(gy[i]),
            da, db);
     if (same) {
-      ga[i] = from_f32<T>(to_f32(from_f32<T>(to_f32(ga[i]) + da)) + db);
+      ga[i] = from_f32<T>(to_f32(from_f32<T>((acc_a ? to_f32(ga[i]) : 0.f) + da)) + db);
     } else {
-      ga[i] = from_f32<T>(to_f32(ga[i]) + da);
-      gb[i] = from_f32<T>(to_f32(gb[i]) + db);
+      ga[i] = from_f32<T>((acc_a ? to_f32(ga[i]) : 0.f) + da);
+      gb[i] = from_f32<T>((acc_b ? to_f32(gb[i]) : 0.f) + db);
     }
   };
   if constexpr (VEC) {
@@ -149,8 +151,9 @@ __global__ __launch_bounds__(kBlock) void binary_bw_flat_kernel(const T *a, cons
       if constexpr (OP::kB) vb = load_pack(b + p * N);
       if constexpr (OP::kY) vy = load_pack(y + p * N);
       const Pack<T> vg = load_pack(gy + p * N);
-      Pack<T> oa = load_pack(ga + p * N), ob;
-      if (!same) ob = load_pack(gb + p * N);
+      Pack<T> oa, ob;
+      if (acc_a) oa = load_pack(ga + p * N);
+      if (!same && acc_b) ob = load_pack(gb + p * N);
 #pragma unroll
       for (int e = 0; e < N; ++e) {
         float av = 0.f, bv = 0.f, yv = 0.f, da, db;
@@ -159,10 +162,10 @@ __global__ __launch_bounds__(kBlock) void binary_bw_flat_kernel(const T *a, cons
         if constexpr (OP::kY) yv = to_f32(vy.v[e]);
         OP::bw(av, bv, yv, to_f32(vg.v[e]), da, db);
         if (same) {
-          oa.v[e] = from_f32<T>(to_f32(from_f32<T>(to_f32(oa.v[e]) + da)) + db);
+          oa.v[e] = from_f32<T>(to_f32(from_f32<T>((acc_a ? to_f32(oa.v[e]) : 0.f) + da)) + db);
         } else {
-          oa.v[e] = from_f32<T>(to_f32(oa.v[e]) + da);
-          ob.v[e] = from_f32<T>(to_f32(ob.v[e]) + db);
+          oa.v[e] = from_f32<T>((acc_a ? to_f32(oa.v[e]) : 0.f) + da);
+          ob.v[e] = from_f32<T>((acc_b ? to_f32(ob.v[e]) : 0.f) + db);
         }
       }
       store_pack(ga + p * N, oa);
@@ -182,11 +185,12 @@ __global__ __launch_bounds__(kBlock) void binary_bw_flat_kernel(const T *a, cons
 // (tx, ty) walks samples ty, ty + TY, ...; it updates the batched operand's
 // gradient in place and keeps the broadcast operand's in registers.  The TY
 // partial sums of an item are then added in order of ty and the total added
-// to the broadcast gradient once.
+// to the broadcast gradient once.  acc_full / acc_one off: the old value of the batched / the
+// broadcast operand's gradient counts as zero and is not read.
 template <typename T, typename OP, bool VEC, int TY>
 __global__ __launch_bounds__(kBlock) void binary_bw_bcast_kernel(const T *a, const T *b, const T *y, const T *gy,
                                                                   T *ga, T *gb, size_t volume, uint32_t bs,
-                                                                  bool a_bcast) {
+                                                                  bool a_bcast, bool acc_full, bool acc_one) {
   constexpr int N = VEC ? Pack<T>::N : 1;
   constexpr int TX = kBlock / TY;
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -209,7 +213,8 @@ __global__ __launch_bounds__(kBlock) void binary_bw_bcast_kernel(const T *a, con
         if constexpr (OP::kB) vb = load_pack(b + ob);
         if constexpr (OP::kY) vy = load_pack(y + offn);
         const Pack<T> vg = load_pack(gy + offn);
-        Pack<T> out = load_pack(gfull);
+        Pack<T> out;
+        if (acc_full) out = load_pack(gfull);
 #pragma unroll
         for (int e = 0; e < N; ++e) {
           float av = 0.f, bv = 0.f, yv = 0.f, da, db;
@@ -218,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void binary_bw_bcast_kernel(const T *a, con
           if constexpr (OP::kY) yv = to_f32(vy.v[e]);
           OP::bw(av, bv, yv, to_f32(vg.v[e]), da, db);
           acc[e] += a_bcast ? da : db;
-          out.v[e] = from_f32<T>(to_f32(out.v[e]) + (a_bcast ? db : da));
+          out.v[e] = from_f32<T>((acc_full ? to_f32(out.v[e]) : 0.f) + (a_bcast ? db : da));
         }
         store_pack(gfull, out);
       } else {
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void binary_bw_bcast_kernel(const T *a, con
         OP::bw(OP::kA ? to_f32(a[oa]) : 0.f, OP::kB ? to_f32(b[ob]) : 0.f, OP::kY ? to_f32(y[offn]) : 0.f,
                to_f32(gy[offn]), da, db);
         acc[0] += a_bcast ? da : db;
-        *gfull = from_f32<T>(to_f32(*gfull) + (a_bcast ? db : da));
+        *gfull = from_f32<T>((acc_full ? to_f32(*gfull) : 0.f) + (a_bcast ? db : da));
       }
     }
   }
@@ -245,12 +250,13 @@ __global__ __launch_bounds__(kBlock) void binary_bw_bcast_kernel(const T *a, con
   if (ty == 0 && live) {
     T *g1 = (a_bcast ? ga : gb) + off1;
     if constexpr (VEC) {
-      Pack<T> out = load_pack(g1);
+      Pack<T> out;
+      if (acc_one) out = load_pack(g1);
 #pragma unroll
-      for (int e = 0; e < N; ++e) out.v[e] = from_f32<T>(to_f32(out.v[e]) + acc[e]);
+      for (int e = 0; e < N; ++e) out.v[e] = from_f32<T>((acc_one ? to_f32(out.v[e]) : 0.f) + acc[e]);
       store_pack(g1, out);
     } else {
-      *g1 = from_f32<T>(to_f32(*g1) + acc[0]);
+      *g1 = from_f32<T>((acc_one ? to_f32(*g1) : 0.f) + acc[0]);
     }
   }
 }
@@ -340,7 +346,7 @@ int launch_scalar_fw(phip_ctx *ctx, int k_on_left, const void *x, const void *k,
 template <typename T, typename OP>
 int launch_binary_bw(phip_ctx *ctx, const void *a, const void *b, const void *y, const void *gy, void *ga, void *gb,
                      uint32_t volume, uint32_t ba, uint32_t bb) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_KEEP_ZEROS(ctx);
   const int rc = check_batches(ba, bb);
   if (rc != PHIP_OK) return rc;
   if (volume == 0) return PHIP_OK;
@@ -348,6 +354,18 @@ int launch_binary_bw(phip_ctx *ctx, const void *a, const void *b, const void *y,
   PHIP_REQUIRE(!OP::kA || a != nullptr, "this gradient needs a");
   PHIP_REQUIRE(!OP::kB || b != nullptr, "this gradient needs b");
   PHIP_REQUIRE(!OP::kY || y != nullptr, "this gradient needs y");
+  PHIP_REQUIRE(ba == bb || ga != gb, "gradients of operands with different batch sizes cannot share memory");
+  // a gradient noted as zero and not yet filled is written instead of added into
+  const size_t na = (size_t)volume * ba * sizeof(T), nb = (size_t)volume * bb * sizeof(T);
+  const size_t ny = na > nb ? na : nb;
+  auto read_too = [&](const void *g, size_t bytes) {
+    return shares_memory(g, bytes, gy, ny) || (OP::kA && shares_memory(g, bytes, a, na)) ||
+           (OP::kB && shares_memory(g, bytes, b, nb)) || (OP::kY && shares_memory(g, bytes, y, ny));
+  };
+  const bool apart = ga == gb || !shares_memory(ga, na, gb, nb);
+  const bool acc_a = !apart || read_too(ga, na) || !zeros_take(ctx, ga, na);
+  const bool acc_b = ga == gb ? acc_a : (!apart || read_too(gb, nb) || !zeros_take(ctx, gb, nb));
+  PHIP_FLUSH_ZEROS(ctx);
   constexpr int N = Pack<T>::N;
   const T *pa = static_cast<const T *>(a);
   const T *pb = static_cast<const T *>(b);
@@ -362,13 +380,12 @@ int launch_binary_bw(phip_ctx *ctx, const void *a, const void *b, const void *y,
     const bool same = ga == gb;
     if (all_aligned) {
       hipLaunchKernelGGL((binary_bw_flat_kernel<T, OP, true>), dim3(blocks_for(n / N + N, ctx)), dim3(kBlock), 0,
-                         ctx->stream, pa, pb, py, pgy, pga, pgb, n, same);
+                         ctx->stream, pa, pb, py, pgy, pga, pgb, n, same, acc_a, acc_b);
     } else {
       hipLaunchKernelGGL((binary_bw_flat_kernel<T, OP, false>), dim3(blocks_for(n, ctx)), dim3(kBlock), 0,
-                         ctx->stream, pa, pb, py, pgy, pga, pgb, n, same);
+                         ctx->stream, pa, pb, py, pgy, pga, pgb, n, same, acc_a, acc_b);
     }
   } else {
-    PHIP_REQUIRE(ga != gb, "gradients of operands with different batch sizes cannot share memory");
     const bool a_bcast = ba == 1;
     const uint32_t bs = a_bcast ? bb : ba;
     const bool vec = all_aligned && volume % N == 0;
@@ -378,7 +395,8 @@ int launch_binary_bw(phip_ctx *ctx, const void *a, const void *b, const void *y,
 #define PHIP_BCAST(VEC, TY)                                                                                       \
   hipLaunchKernelGGL((binary_bw_bcast_kernel<T, OP, VEC, TY>),                                                    \
                      dim3((unsigned)((items + kBlock / TY - 1) / (kBlock / TY))), dim3(kBlock), 0, ctx->stream,   \
-                     pa, pb, py, pgy, pga, pgb, (size_t)volume, bs, a_bcast)
+                     pa, pb, py, pgy, pga, pgb, (size_t)volume, bs, a_bcast, a_bcast ? acc_b : acc_a,                \
+                     a_bcast ? acc_a : acc_b)
     if (vec && deep) PHIP_BCAST(true, 8);
     else if (vec) PHIP_BCAST(true, 1);
     else if (deep) PHIP_BCAST(false, 8);

@@ -174,16 +174,16 @@ __global__ __launch_bounds__(kBlock) void map_fw_kernel(const F f, const T *x, T
   }
 }
 
-// gx[i] += f.bw(x[i], y[i], gy[i]).
+// gx[i] += f.bw(x[i], y[i], gy[i]).  `accumulate` off: gx's old value counts as zero and is not read.
 template <typename T, typename F, bool VEC>
 __global__ __launch_bounds__(kBlock) void map_bw_kernel(const F f, const T *x, const T *y, const T *gy, T *gx,
-                                                         size_t n) {
+                                                         size_t n, bool accumulate) {
   const size_t stride = (size_t)gridDim.x * kBlock;
   const size_t first = (size_t)blockIdx.x * kBlock + threadIdx.x;
   auto one = [&](size_t i) {
     const float xv = F::kX ? to_f32(x[i]) : 0.f;
     const float yv = F::kY ? to_f32(y[i]) : 0.f;
-    gx[i] = from_f32<T>(to_f32(gx[i]) + f.bw(xv, yv, to_f32(gy[i])));
+    gx[i] = from_f32<T>((accumulate ? to_f32(gx[i]) : 0.f) + f.bw(xv, yv, to_f32(gy[i])));
   };
   if constexpr (VEC) {
     constexpr int N = Pack<T>::N;
@@ -193,13 +193,14 @@ __global__ __launch_bounds__(kBlock) void map_bw_kernel(const F f, const T *x, c
       if constexpr (F::kX) px = load_pack(x + p * N);
       if constexpr (F::kY) py = load_pack(y + p * N);
       const Pack<T> pg = load_pack(gy + p * N);
-      Pack<T> acc = load_pack(gx + p * N);
+      Pack<T> acc;
+      if (accumulate) acc = load_pack(gx + p * N);
 #pragma unroll
       for (int e = 0; e < N; ++e) {
         float xv = 0.f, yv = 0.f;
         if constexpr (F::kX) xv = to_f32(px.v[e]);
         if constexpr (F::kY) yv = to_f32(py.v[e]);
-        acc.v[e] = from_f32<T>(to_f32(acc.v[e]) + f.bw(xv, yv, to_f32(pg.v[e])));
+        acc.v[e] = from_f32<T>((accumulate ? to_f32(acc.v[e]) : 0.f) + f.bw(xv, yv, to_f32(pg.v[e])));
       }
       store_pack(gx + p * N, acc);
     }
@@ -240,11 +241,17 @@ int launch_fw(phip_ctx *ctx, const F &f, const void *x, void *y, size_t n) {
 
 template <typename T, typename F>
 int launch_bw(phip_ctx *ctx, const F &f, const void *x, const void *y, const void *gy, void *gx, size_t n) {
-  PHIP_ENTER(ctx);
+  PHIP_ENTER_KEEP_ZEROS(ctx);
   if (n == 0) return PHIP_OK;
   PHIP_REQUIRE(gy != nullptr && gx != nullptr, "null pointer");
   PHIP_REQUIRE(!F::kX || x != nullptr, "this gradient needs x");
   PHIP_REQUIRE(!F::kY || y != nullptr, "this gradient needs y");
+  // gx noted as zero and not yet filled: write instead of add
+  const size_t bytes = n * sizeof(T);
+  const bool read_too = shares_memory(gx, bytes, gy, bytes) || (F::kX && shares_memory(gx, bytes, x, bytes)) ||
+                        (F::kY && shares_memory(gx, bytes, y, bytes));
+  const bool accumulate = read_too || !zeros_take(ctx, gx, bytes);
+  PHIP_FLUSH_ZEROS(ctx);
   const T *px = static_cast<const T *>(x);
   const T *py = static_cast<const T *>(y);
   const T *pgy = static_cast<const T *>(gy);
@@ -252,10 +259,10 @@ int launch_bw(phip_ctx *ctx, const F &f, const void *x, const void *y, const voi
   const bool vec = aligned16(gy) && aligned16(gx) && (!F::kX || aligned16(x)) && (!F::kY || aligned16(y));
   if (vec) {
     hipLaunchKernelGGL((map_bw_kernel<T, F, true>), dim3(blocks_for(n / Pack<T>::N + Pack<T>::N, ctx)),
-                       dim3(kBlock), 0, ctx->stream, f, px, py, pgy, pgx, n);
+                       dim3(kBlock), 0, ctx->stream, f, px, py, pgy, pgx, n, accumulate);
   } else {
     hipLaunchKernelGGL((map_bw_kernel<T, F, false>), dim3(blocks_for(n, ctx)), dim3(kBlock), 0, ctx->stream, f,
-                       px, py, pgy, pgx, n);
+                       px, py, pgy, pgx, n, accumulate);
   }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;

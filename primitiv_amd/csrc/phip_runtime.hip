@@ -1,5 +1,6 @@
 // Contexts, the device memory pool, copies, events and the host randomizer.
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <random>
 #include <cmath>
@@ -52,7 +53,7 @@ static int fixed_scratch_of(int device, unsigned char **out) {
 }
 
 static int pool_alloc_from(phip_ctx *ctx, Pool &pool, size_t bytes, void **out, size_t *allocated);
-static int pool_free_locked(Pool &pool, void *ptr);
+static int pool_free_locked(phip_ctx *ctx, Pool &pool, void *ptr);
 
 int scratch_alloc(phip_ctx *ctx, size_t bytes, void **out) {
   if (!ctx->fixed_mode) return pool_alloc_from(ctx, ctx->scratch_pool, bytes, out, nullptr);
@@ -73,7 +74,7 @@ void scratch_free(phip_ctx *ctx, void *ptr) {
   const unsigned char *p = static_cast<const unsigned char *>(ptr);
   if (ctx->fixed_scratch && p >= ctx->fixed_scratch && p < ctx->fixed_scratch + kFixedTicketBytes + kFixedScratchBytes) return;
   std::lock_guard<std::mutex> lock(ctx->mutex);
-  (void)pool_free_locked(ctx->scratch_pool, ptr);
+  (void)pool_free_locked(ctx, ctx->scratch_pool, ptr);
 }
 
 uint32_t *tile_tickets(phip_ctx *ctx) {
@@ -115,11 +116,43 @@ static void release_reserved_on_device(int device) {
   }
 }
 
-static int pool_free_locked(Pool &pool, void *ptr) {
+static void zeros_drop_locked(phip_ctx *ctx, const void *p, size_t bytes) {
+  if (ctx->zeros.empty()) return;
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(p), hi = lo + bytes;
+  size_t kept = 0;
+  for (const PendingZero &z : ctx->zeros) {
+    if (!(z.lo >= lo && z.lo + z.bytes <= hi)) ctx->zeros[kept++] = z;
+  }
+  ctx->zeros.resize(kept);
+  ctx->zeros_count.store((int)kept, std::memory_order_relaxed);
+}
+
+void zeros_drop(phip_ctx *ctx, const void *p, size_t bytes) {
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  zeros_drop_locked(ctx, p, bytes);
+}
+
+bool zeros_take(phip_ctx *ctx, const void *p, size_t bytes) {
+  if (ctx->zeros_count.load(std::memory_order_relaxed) == 0) return false;
+  std::lock_guard<std::mutex> lock(ctx->mutex);
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+  for (size_t i = 0; i < ctx->zeros.size(); ++i) {
+    if (ctx->zeros[i].lo == lo && ctx->zeros[i].bytes == bytes) {
+      ctx->zeros.erase(ctx->zeros.begin() + (long)i);
+      ctx->zeros_count.store((int)ctx->zeros.size(), std::memory_order_relaxed);
+      return true;
+    }
+  }
+  return false;
+}
+
+static int pool_free_locked(phip_ctx *ctx, Pool &pool, void *ptr) {
   auto it = pool.supplied.find(ptr);
   if (it == pool.supplied.end()) {
     return fail(PHIP_ERR_INVALID_ARGUMENT, "Detected to dispose unknown handle: %p", ptr);
   }
+  // whatever the block was to be filled with no longer matters
+  zeros_drop_locked(ctx, ptr, (size_t)1 << it->second);
   pool.reserved[it->second].push_back(ptr);
   pool.supplied.erase(it);
   return PHIP_OK;
@@ -193,6 +226,11 @@ int ctx_create(int device_id, bool with_lanes, phip_ctx **out) {
     delete ctx;
     return fail(PHIP_ERR_RUNTIME, "context creation failed: %s", hipGetErrorString(e));
   }
+  {
+    const char *v = std::getenv("PHIP_DEFER_ZERO_FILLS");
+    ctx->defer_zero_fills = !(v != nullptr && v[0] == '0');
+    ctx->zeros.reserve(16);
+  }
   ctx->id = phip::g_next_id.fetch_add(1);
   {
     std::lock_guard<std::mutex> lock(phip::g_registry_mutex);
@@ -262,6 +300,11 @@ int phip_ctx_destroy(phip_ctx *ctx) {
     phip::g_registry.erase(ctx->id);
   }
   int rc = lanes_rc;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->zeros.clear();  // fills nobody will read
+    ctx->zeros_count.store(0, std::memory_order_relaxed);
+  }
   if (hipSetDevice(ctx->device) != hipSuccess ||
       hipStreamSynchronize(ctx->stream) != hipSuccess) {
     rc = fail(PHIP_ERR_RUNTIME, "synchronisation failed while destroying the context");
@@ -337,6 +380,12 @@ int phip_set_deterministic(phip_ctx *ctx, int on) {
   return PHIP_OK;
 }
 
+int phip_set_deferred_zero_fill(phip_ctx *ctx, int on) {
+  PHIP_ENTER(ctx);  // launches what is noted
+  ctx->defer_zero_fills = on != 0;
+  return PHIP_OK;
+}
+
 int phip_sync(phip_ctx *ctx) {
   PHIP_ENTER_BLOCKING(ctx);
   PHIP_HIP(hipStreamSynchronize(ctx->stream));
@@ -369,6 +418,7 @@ int phip_malloc(phip_ctx *ctx, size_t bytes, void **out) {
 int phip_free(phip_ctx *ctx, void *ptr) {
   PHIP_ENTER_HOST(ctx);
   if (ptr == nullptr) return PHIP_OK;
+  PHIP_FLUSH_ZEROS(ctx);  // a noted fill of this memory must not be launched after it is gone
   PHIP_HIP(hipFree(ptr));
   return PHIP_OK;
 }
@@ -385,7 +435,7 @@ int phip_pool_free(phip_ctx *ctx, void *ptr) {
   PHIP_REQUIRE(ctx != nullptr, "null context");
   if (ptr == nullptr) return PHIP_OK;
   std::lock_guard<std::mutex> lock(ctx->mutex);
-  return phip::pool_free_locked(ctx->pool, ptr);
+  return phip::pool_free_locked(ctx, ctx->pool, ptr);
 }
 
 int phip_pool_free_by_id(uint64_t ctx_id, void *ptr) {
@@ -394,7 +444,7 @@ int phip_pool_free_by_id(uint64_t ctx_id, void *ptr) {
   auto it = phip::g_registry.find(ctx_id);
   if (it == phip::g_registry.end()) return PHIP_OK;  // pool already gone
   std::lock_guard<std::mutex> lock(it->second->mutex);
-  return phip::pool_free_locked(it->second->pool, ptr);
+  return phip::pool_free_locked(it->second, it->second->pool, ptr);
 }
 
 int phip_pool_release_reserved(phip_ctx *ctx) {
@@ -478,6 +528,7 @@ int phip_event_destroy(phip_event *ev) {
 
 int phip_event_record(phip_ctx *ctx, phip_event *ev) {
   PHIP_ENTER_HOST(ctx);
+  PHIP_FLUSH_ZEROS(ctx);
   PHIP_REQUIRE(ev != nullptr, "null event");
   if (ctx->lanes != nullptr) {
     const int rc = phip::lanes_order_main_after_side(ctx);

@@ -421,6 +421,11 @@ class HIP:
         default); off: every launch on one stream."""
         _lib.call("phip_set_overlap", self._ctx, 1 if on else 0)
 
+    def set_deferred_zero_fill(self, on=True):
+        """Zero fills are noted and folded into the gradient operation that follows (the default);
+        off: every fill is launched when it is asked for."""
+        _lib.call("phip_set_deferred_zero_fill", self._ctx, 1 if on else 0)
+
     def gemm_trace(self, on=True):
         """Names of the GEMM kernels that this device's matmul calls went to since the previous call
         (a list, launch order per stream); `on` switches the note-taking on or off from here on."""
