@@ -131,6 +131,7 @@ def _native():
         l.phip_bench_front_loop.argtypes = [vp, i, vp, vp, pp, pp, ctypes.POINTER(_Dims), i, i, i] + out
         l.phip_bench_lstm_loop.argtypes = [vp, i, ctypes.POINTER(_LstmDims), vp, vp, vp, vp, pp, pp, vp, vp, i, i, i] + out
         l.phip_bench_raw_loop.restype = l.phip_bench_front_loop.restype = l.phip_bench_lstm_loop.restype = i
+        l.phip_bench_last_enqueue_ms.restype = ctypes.c_double
         _bench_lib = l
     return _bench_lib
 
@@ -588,7 +589,9 @@ def measure_lstm(storage, steps, warmup, hidden=650, batch=64, timesteps=35):
         _timed_native(loop(False), max(2, warmup), 0)
         fw_ms, fw_host = _timed_native(loop(True), steps, 1)
         all_ms, all_host = _timed_native(loop(False), steps, 1)
+        enqueue = L.phip_bench_last_enqueue_ms() / steps
         out[key] = {"us_per_timestep_forward": fw_ms * 1e3 / T, "us_per_timestep_forward_backward": all_ms * 1e3 / T,
+                    "us_per_timestep_forward_backward_host_enqueue_only": enqueue * 1e3 / T,
                     "us_per_timestep_forward_backward_host_clock": all_host * 1e3 / T,
                     "us_per_timestep_forward_host_clock": fw_host * 1e3 / T}
     flops = 3 * 2 * (4 * H) * (I + H) * B

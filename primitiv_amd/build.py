@@ -30,6 +30,7 @@ SOURCES = [
     "phip_gemm_f32_stream_pair.hip",
     "phip_conv_pool.hip",
     "phip_gemm_h16.hip",
+    "phip_gemm_h16_skinny.hip",
     "phip_gemm_h16_big.hip",
     "phip_matmul.hip",
 ]

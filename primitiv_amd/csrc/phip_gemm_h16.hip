@@ -485,7 +485,9 @@ int gemm_h16_typed(phip_ctx *ctx, const Gemm &p) {
 int gemm_h16(phip_ctx *ctx, const Gemm &p, Elem elem) {
   if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return PHIP_OK;
   bool handled = false;
-  const int rc = gemm_h16_big(ctx, p, elem, &handled);
+  int rc = gemm_h16_skinny(ctx, p, elem, &handled);
+  if (rc != PHIP_OK || handled) return rc;
+  rc = gemm_h16_big(ctx, p, elem, &handled);
   if (rc != PHIP_OK || handled) return rc;
   return elem == Elem::BF16 ? gemm_h16_typed<true>(ctx, p) : gemm_h16_typed<false>(ctx, p);
 }

@@ -79,7 +79,7 @@ struct phip_ctx {
   std::mutex mutex;  // guards `pool` and `scratch_pool`
   // Kernels whose dynamic-LDS limit has been raised on this context's device
   // (one bit per kernel, see phip::raise_lds_limit).
-  uint32_t lds_limit_raised = 0;
+  uint64_t lds_limit_raised = 0;
   // One counter per output tile of a launch whose workgroups share tiles (see
   // phip::kTicketSlots); all zero between launches.
   uint32_t *tile_tickets = nullptr;
@@ -244,14 +244,15 @@ enum LdsSlot {
   kSlotGemmF32RankK = 21, // 1
   kSlotGemmF32StreamPair = 22,  // 1
   kSlotGemmH16Mid = 23,   // 6
+  kSlotGemmH16Skinny = 29,  // 8
 };
 
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on
-// the context's device; done once per context and kernel (`slot` < 32).
+// the context's device; done once per context and kernel (`slot` < 64).
 inline int raise_lds_limit(phip_ctx *ctx, int slot, const void *kernel, int bytes) {
-  if (ctx->lds_limit_raised & (1u << slot)) return PHIP_OK;
+  if (ctx->lds_limit_raised & (1ull << slot)) return PHIP_OK;
   PHIP_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-  ctx->lds_limit_raised |= 1u << slot;
+  ctx->lds_limit_raised |= 1ull << slot;
   return PHIP_OK;
 }
 
@@ -306,6 +307,10 @@ int gemm_f32_stream_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, b
 constexpr long kStreamedOperandBytes = 8L << 20;
 int gemm_h16(phip_ctx *ctx, const Gemm &g, Elem elem);
 int gemm_h16_big(phip_ctx *ctx, const Gemm &g, Elem elem, bool *handled);
+// 16-bit products with a narrow side or a short K (per-timestep shapes); the pair: both gradient products
+// of one matmul_bw call in one launch.
+int gemm_h16_skinny(phip_ctx *ctx, const Gemm &g, Elem elem, bool *handled);
+int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, Elem elem, bool *handled);
 
 }  // namespace phip
 

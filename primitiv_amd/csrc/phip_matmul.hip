@@ -185,6 +185,15 @@ static int matmul_bw(phip_ctx *ctx, Elem elem, const void *a, const void *b, con
       if (rc != PHIP_OK || handled) return rc;
     }
   }
+  if (elem != Elem::F32) {
+    const char *ga0 = static_cast<const char *>(ga), *gb0 = static_cast<const char *>(gb);
+    const size_t ga_bytes = 2 * (size_t)di * dj * ba, gb_bytes = 2 * (size_t)dj * dk * bb;
+    if (ga0 + ga_bytes <= gb0 || gb0 + gb_bytes <= ga0) {
+      bool handled = false;
+      rc = gemm_h16_skinny_pair(ctx, p, q, elem, &handled);
+      if (rc != PHIP_OK || handled) return rc;
+    }
+  }
   rc = gemm_dispatch(ctx, p, elem);
   if (rc != PHIP_OK) return rc;
   return gemm_dispatch(ctx, q, elem);

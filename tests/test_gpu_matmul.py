@@ -555,6 +555,61 @@ def test_long_k_few_tiles_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
         assert norm_rel_err(got, ref) <= ulp
 
 
+# The per-timestep shapes on the 16-bit devices: a narrow side (the minibatch) against a weight
+# matrix, forward and both gradients - the streamed-operand and paired-gradient lists of the fp32
+# device, plus rows that are not 16-byte aligned (650, 1300, 518 columns of 16-bit values), ragged
+# M / N / K, a minibatch of 1 and of 100, per-sample operands, a contraction over the minibatch.
+# Inputs are exactly representable, so what is left is the one rounding of each output.
+SKINNY_H16 = [  # di, dj, dk, ba, bb
+    (10000, 650, 1, 1, 64),     # output projection
+    (2048, 512, 1, 1, 64),      # recurrent gate
+    (2600, 1300, 1, 1, 64),     # an LSTM layer with 650 hidden units
+    (2600, 1300, 1, 1, 20),
+    (256, 784, 1, 1, 128),      # dense layer
+    (4100, 518, 1, 1, 40),
+    (4100, 520, 2, 1, 30),
+    (2052, 516, 1, 1, 60),
+    (1028, 512, 48, 5, 1),      # the shared operand on the right: contraction over the minibatch
+    (132, 260, 24, 6, 6),       # per-sample products
+    (8192, 260, 1, 1, 1),
+    (70, 3000, 40, 1, 1),       # long K, one tile
+    (66, 70, 34, 1, 3),         # everything ragged and small
+    (64, 64, 64, 1, 1),
+    (800, 784, 1, 1, 100),
+    (10, 800, 1, 1, 100),       # ten output rows
+]
+
+
+@pytest.mark.parametrize("which", ["f16", "bf16"])
+@pytest.mark.parametrize("di,dj,dk,ba,bb", SKINNY_H16)
+def test_per_timestep_shapes_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
+    d = dev16 if which == "f16" else devbf16
+    rng = np.random.default_rng(di + 3 * dj + dk + ba)
+    bs = max(ba, bb)
+    r16 = (lambda x: x.astype(np.float16).astype(np.float32)) if which == "f16" else \
+        (lambda x: (x.view(np.uint32) & 0xFFFF0000).view(np.float32))
+    a = r16(rng.standard_normal(di * dj * ba).astype(np.float32))
+    b = r16(rng.standard_normal(dj * dk * bb).astype(np.float32))
+    gy = r16(rng.standard_normal(di * dk * bs).astype(np.float32))
+    ga0 = r16(rng.standard_normal(a.size).astype(np.float32))
+    gb0 = r16(rng.standard_normal(b.size).astype(np.float32))
+    d.gemm_trace(True)
+    y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    kernels = d.gemm_trace(False)
+    if dj % 2 == 0 and di % 2 == 0:          # the kernel this list is for
+        assert kernels[0].startswith("h16_skinny"), kernels
+        # (a contraction over fewer than 16 values, e.g. the weight gradient of a minibatch of one, is left to the staged kernel)
+        assert min(di, dj, dk * bb) < 16 or all(k.startswith("h16_skinny") for k in kernels), kernels
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    ulp = 2.0 ** -10 if which == "f16" else 2.0 ** -7
+    for name, got, ref in (("y", y, ry), ("ga", ga, rga), ("gb", gb, rgb)):
+        assert norm_rel_err(got, ref) <= ulp, name
+    # again, over pool memory that holds the first call's results: an overwriting product must not add
+    y2, ga2, gb2 = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    assert np.array_equal(y2, y) and np.array_equal(ga2, ga) and np.array_equal(gb2, gb)     # and the same bits
+
+
 def test_f16_matches_oracle_on_rounded_inputs(dev16):
     # With inputs already representable in fp16 the only error left is the
     # final rounding of the output (<= 2^-11 relative per element) on top of
