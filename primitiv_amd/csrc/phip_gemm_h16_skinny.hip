@@ -163,6 +163,43 @@ __device__ inline uint4v keep_first(uint4v f, int valid) {
   return r;
 }
 
+// 16 bytes to / from memory at device scope (past the per-XCD L2s), as the partial tiles of a split
+// product travel.  The loads are not tracked by the compiler: the caller waits (wait_loads) before it
+// reads what they return.
+// (A store of more than 8 bytes reads its data registers a little after it has issued; the compiler keeps
+// the next write of those registers away from stores it knows, the wait states here do it for this one.)
+__device__ inline void store_device_scope(float *p, float4v v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
+}
+// The four 16-byte pieces (1 KiB apart) of each of four partial tiles, all sixteen loads in flight at
+// once, and the wait for them, in one statement: the compiler sees values that are there.
+__device__ inline void load_four_tiles_device_scope(float4v (&v)[4][4], const float *q0, const float *q1,
+                                                    const float *q2, const float *q3) {
+  asm volatile(
+      "global_load_dwordx4 %0, %16, off sc1\n\t"
+      "global_load_dwordx4 %1, %16, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %2, %16, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %3, %16, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %4, %17, off sc1\n\t"
+      "global_load_dwordx4 %5, %17, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %6, %17, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %7, %17, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %8, %18, off sc1\n\t"
+      "global_load_dwordx4 %9, %18, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %10, %18, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %11, %18, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %12, %19, off sc1\n\t"
+      "global_load_dwordx4 %13, %19, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %14, %19, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %15, %19, off offset:3072 sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(v[0][0]), "=&v"(v[0][1]), "=&v"(v[0][2]), "=&v"(v[0][3]), "=&v"(v[1][0]), "=&v"(v[1][1]), "=&v"(v[1][2]),
+        "=&v"(v[1][3]), "=&v"(v[2][0]), "=&v"(v[2][1]), "=&v"(v[2][2]), "=&v"(v[2][3]), "=&v"(v[3][0]), "=&v"(v[3][1]),
+        "=&v"(v[3][2]), "=&v"(v[3][3])
+      : "v"(q0), "v"(q1), "v"(q2), "v"(q3)
+      : "memory");
+}
+
 template <bool BF16>
 __device__ inline float4v mfma(uint4v a, uint4v b, float4v c) {
   if constexpr (BF16) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c, 0, 0, 0);
@@ -276,13 +313,13 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
   if (g.splits > 1) {
     const long tile_id = ((long)z * g.tiles_n + tile_n) * g.tiles_m + tile_m;
     float *P = g.partial + (tile_id * g.splits + split) * (long)(TM * TN) + wave * 1024 + lane * 4;
+    // the stores below are assembly that the compiler does not look into: it would not keep the distance
+    // that a matrix instruction's result needs before a memory instruction reads it
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          __hip_atomic_store(P + (i * 2 + j) * 256 + v, acc[i][j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int j = 0; j < 2; ++j) store_device_scope(P + (i * 2 + j) * 256, acc[i][j]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own stores acknowledged before the ticket
     __syncthreads();
     if (tid == 0) {
@@ -298,20 +335,18 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
-    for (int r0 = 0; r0 < g.splits; r0 += 2) {
-      float part[2][16];
+    // four ranges at a time: sixteen 16-byte loads in flight per lane, added in the order of the ranges
+    for (int r0 = 0; r0 < g.splits; r0 += 4) {
+      float4v part[4][4];
+      const float *q[4];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const float *q = Q + (long)(r0 + u < g.splits ? r0 + u : r0) * (TM * TN);
+      for (int u = 0; u < 4; ++u) q[u] = Q + (long)(r0 + u < g.splits ? r0 + u : r0) * (TM * TN);
+      load_four_tiles_device_scope(part, q[0], q[1], q[2], q[3]);
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          part[u][e] = __hip_atomic_load(q + (e >> 2) * 256 + (e & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 4; ++u)
         if (r0 + u < g.splits) {
 #pragma unroll
-          for (int e = 0; e < 16; ++e) acc[(e >> 2) >> 1][(e >> 2) & 1][e & 3] += part[u][e];
+          for (int e = 0; e < 4; ++e) acc[e >> 1][e & 1] += part[u][e];
         }
     }
   }
@@ -404,8 +439,8 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
 
   // Stages per workgroup: the choice that a small cost model likes best (microseconds): the loads of the
   // workgroups that share a compute unit (about 0.4 per 16 KiB K tile), the exchange of partial tiles when
-  // K is cut (a round trip through memory, longer with more ranges), and a second round of workgroups if
-  // the grid does not fit the chip at once.
+  // K is cut (store, ticket, then one round trip through memory per four ranges), and a second round of
+  // workgroups if the grid does not fit the chip at once.
   int best_s = 0;
   double best = 0.0;
   for (int s = 1; s <= kMaxStages; ++s) {
@@ -413,7 +448,7 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
     const int s_eff = (int)((total_ktiles + splits - 1) / splits);
     if (s_eff != s && s != kMaxStages) continue;  // the same cut as a smaller s
     int occ = (160 * 1024) / (s_eff * kStage);
-    if (occ > 6) occ = 6;  // 80 registers per lane: six wavefronts per SIMD
+    if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
     if (places_per_cu > 0 && occ > places_per_cu) occ = places_per_cu;
     if (occ < 1) continue;
     const long grid = tiles * splits;
@@ -423,7 +458,7 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
     const long rounds = (grid + places - 1) / places;
     long per_cu = (grid + cus - 1) / cus;
     if (per_cu > occ) per_cu = occ;
-    const double cost = rounds * (1.0 + 0.4 * s_eff * per_cu) + (splits > 1 ? 1.5 + 0.05 * splits : 0.0);
+    const double cost = rounds * (1.0 + 0.4 * s_eff * per_cu) + (splits > 1 ? 2.0 + 1.2 * ((splits + 3) / 4) : 0.0);
     if (best_s == 0 || cost < best) {
       best = cost;
       best_s = s_eff;
@@ -522,7 +557,7 @@ int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, E
   const int stages = p1.stages > p2.stages ? p1.stages : p2.stages;
   const int cus = ctx->prop.multiProcessorCount;
   int occ = (160 * 1024) / (stages * kStage);
-  if (occ > 6) occ = 6;  // 80 registers per lane: six wavefronts per SIMD
+  if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
   if (p1.grid + p2.grid > (long)cus * occ) return PHIP_OK;  // would take a second round: two launches do as well
   // the second problem's workgroups start at a multiple of 8, so that both meet the XCDs in order
   const long first_blocks = (p1.grid + 7) / 8 * 8;
