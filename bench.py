@@ -326,9 +326,8 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False, 
         two_front, one_front = (other_front, out["ms_per_step_front"]) if not lanes_for_record else (out["ms_per_step_front"], other_front)
         out["ms_per_step_in_order"], out["ms_per_step_front_in_order"] = one, one_front
         out["frac_binding_roofline_in_order"] = _figures(w, one * 1e-3)["frac_binding_roofline"]
-        if w.storage == "f32":      # 16-bit products always run in order
-            out["ms_per_step_two_lanes"], out["ms_per_step_front_two_lanes"] = two, two_front
-            out["frac_binding_roofline_two_lanes"] = _figures(w, two * 1e-3)["frac_binding_roofline"]
+        out["ms_per_step_two_lanes"], out["ms_per_step_front_two_lanes"] = two, two_front
+        out["frac_binding_roofline_two_lanes"] = _figures(w, two * 1e-3)["frac_binding_roofline"]
     if per_timestep and w.storage == "f32" and not deterministic:
         dev.set_deterministic(True)
         loops.raw(max(2, warmup), 0)

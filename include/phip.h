@@ -108,8 +108,8 @@ int phip_set_deterministic(phip_ctx *ctx, int on);
  * with the sixth such call in a row and goes out of use with the first
  * operation of another kind that enqueues work; phip_fill_f32 counts as a
  * matmul call here (a backward pass resets every gradient before it adds
- * products into it).  Products of more than 4 GFLOP, 16-bit storage and
- * allocation-free calls always run in order.  on == 0 puts every launch back
+ * products into it).  Products of more than 4 GFLOP and allocation-free calls
+ * always run in order.  on == 0 puts every launch back
  * on one stream; the environment variable PHIP_OVERLAP=0 makes that the
  * default of contexts created afterwards.  The call itself waits for neither
  * lane on the host. */

@@ -113,14 +113,10 @@ static int fill_now(phip_ctx *ctx, void *p, float value, size_t n) {
   // A fill is the one operation that sits between the matrix products of a backward pass (every
   // gradient is reset before products are added into it) and it names its memory as they do: it
   // takes a lane like a product instead of releasing the lanes (phip_lanes.hip).
-  // (fp32 only: the products of 16-bit storage never leave the main lane.)
-  if (sizeof(T) == sizeof(float)) {
+  {
     const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
     const phip::MemRange written = {lo, lo + n * sizeof(T), true};
     const int rc = phip::lanes_place(ctx, &written, 1, n * sizeof(T) <= ((size_t)64 << 20), &ctx);
-    if (rc != PHIP_OK) return rc;
-  } else if (ctx->lanes != nullptr) {
-    const int rc = phip::lanes_join(ctx);
     if (rc != PHIP_OK) return rc;
   }
   if (reinterpret_cast<uintptr_t>(p) % 16 == 0) {

@@ -399,13 +399,16 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_skinny_kernel(const SkinnyA
 // Both gradient products of one matmul_bw call in one grid: workgroups below `first` run ga += gy . b^T
 // (operands contiguous along m and n), the others gb += a^T . gy (both contiguous along k).  Per-timestep
 // launches are mostly fixed latency; the two products share it.
+// The second problem's workgroups start at `second_at`, a multiple of 8, so that both problems meet the XCDs
+// in the order their tile numbering expects; workgroups between the two do nothing.
 template <bool BF16>
-__global__ __launch_bounds__(kThreads) void gemm_h16_skinny_pair_kernel(const SkinnyArgs g1, const SkinnyArgs g2, int first) {
+__global__ __launch_bounds__(kThreads) void gemm_h16_skinny_pair_kernel(const SkinnyArgs g1, const SkinnyArgs g2, int first,
+                                                                         int second_at) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_skinny[];
   __shared__ uint32_t flag;
   const int bid = blockIdx.x;
   if (bid < first) skinny_tile<false, false, BF16>(g1, lds_skinny, &flag, bid, first);
-  else skinny_tile<true, true, BF16>(g2, lds_skinny, &flag, bid - first, (int)gridDim.x - first);
+  else if (bid >= second_at) skinny_tile<true, true, BF16>(g2, lds_skinny, &flag, bid - second_at, (int)gridDim.x - second_at);
 }
 
 struct SkinnyPlan {
@@ -558,10 +561,8 @@ int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, E
   const int cus = ctx->prop.multiProcessorCount;
   int occ = (160 * 1024) / (stages * kStage);
   if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
-  if (p1.grid + p2.grid > (long)cus * occ) return PHIP_OK;  // would take a second round: two launches do as well
-  // the second problem's workgroups start at a multiple of 8, so that both meet the XCDs in order
-  const long first_blocks = (p1.grid + 7) / 8 * 8;
-  if (first_blocks != p1.grid) return PHIP_OK;  // (kept simple: the first grid has to be a multiple of 8)
+  const long second_at = (p1.grid + 7) / 8 * 8;
+  if (second_at + p2.grid > (long)cus * occ) return PHIP_OK;  // would take a second round: two launches do as well
   void *b1 = nullptr, *b2 = nullptr;
   int rc = prepare_exchange(ctx, &p1, &b1);
   if (rc == PHIP_OK) rc = prepare_exchange(ctx, &p2, &b2);
@@ -572,15 +573,15 @@ int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, E
   }
   if (rc == PHIP_OK) {
     const int lds = stages * kStage;
-    const unsigned grid = (unsigned)(p1.grid + p2.grid);
+    const unsigned grid = (unsigned)(second_at + p2.grid);
     if (elem == Elem::BF16) {
       auto kern = gemm_h16_skinny_pair_kernel<true>;
       rc = raise_lds(ctx, kSlotGemmH16Skinny + 7, kern, lds);
-      if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, ctx->stream, p1.a, p2.a, (int)p1.grid);
+      if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, ctx->stream, p1.a, p2.a, (int)p1.grid, (int)second_at);
     } else {
       auto kern = gemm_h16_skinny_pair_kernel<false>;
       rc = raise_lds(ctx, kSlotGemmH16Skinny + 6, kern, lds);
-      if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, ctx->stream, p1.a, p2.a, (int)p1.grid);
+      if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, ctx->stream, p1.a, p2.a, (int)p1.grid, (int)second_at);
     }
   }
   if (b1) scratch_free(ctx, b1);

@@ -48,7 +48,8 @@ static MemRange range_of(const void *p, uint64_t elements, Elem elem, bool write
 static int place(phip_ctx *ctx, Elem elem, const MemRange *ranges, int n, uint32_t di, uint32_t dj, uint32_t dk,
                  uint32_t ba, uint32_t bb, phip_ctx **run_on) {
   const double flop = 2.0 * di * dj * dk * (ba > bb ? ba : bb);
-  const bool may_overlap = elem == Elem::F32 && !ctx->fixed_mode && flop <= kMaxOverlapFlop;
+  (void)elem;
+  const bool may_overlap = !ctx->fixed_mode && flop <= kMaxOverlapFlop;
   return lanes_place(ctx, ranges, n, may_overlap, run_on);
 }
 

@@ -17,13 +17,13 @@ pytestmark = pytest.mark.gpu
 S = pa.Shape
 
 
-def _device(overlap, deterministic=True):
+def _device(overlap, deterministic=True, storage="f32"):
     # the library engages its second lane only in a long run of matmul calls and backs off when a run
     # was short; here it is engaged by the first call, every time (read when the context is created)
     saved = {k: os.environ.get(k) for k in ("PHIP_OVERLAP_AFTER", "PHIP_OVERLAP_BACKOFF")}
     os.environ["PHIP_OVERLAP_AFTER"], os.environ["PHIP_OVERLAP_BACKOFF"] = "1", "0"
     try:
-        d = pa.HIP(0)
+        d = pa.HIP(0) if storage == "f32" else pa.HIP16(0, storage=storage)
     finally:
         for k, v in saved.items():
             if v is None:
@@ -35,11 +35,11 @@ def _device(overlap, deterministic=True):
     return d
 
 
-def _run_both(program, deterministic=True):
+def _run_both(program, deterministic=True, storage="f32"):
     """program(dev) -> list of numpy arrays; returns (with lanes, in order)."""
     out = []
     for overlap in (True, False):
-        d = _device(overlap, deterministic)
+        d = _device(overlap, deterministic, storage)
         try:
             out.append([np.asarray(v, dtype=np.float32) for v in program(d)])
         finally:
@@ -340,3 +340,38 @@ def test_scratch_of_a_split_product_never_becomes_a_tensor_of_the_other_lane():
     want = oracle.matmul_fw(a, b, m, k, n, 1, 1)
     for i in range(0, len(in_order), 3):
         assert norm_rel_err(lanes[i], want) <= 1e-4 and norm_rel_err(lanes[i + 1], want) <= 1e-4
+
+
+@pytest.mark.parametrize("storage", ["f16", "bf16"])
+@pytest.mark.parametrize("m,k,n", [(2048, 512, 64), (1000, 650, 64), (96, 200, 16)])
+def test_sixteen_bit_products_on_two_lanes(storage, m, k, n):
+    # the per-timestep products of the 16-bit devices take lanes like the fp32 ones: forward products that
+    # feed one another, gradients accumulated by calls on different lanes, gradients reset per timestep
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal(m * k).astype(np.float32) / np.sqrt(k)
+    at = rng.standard_normal(k * m).astype(np.float32) / np.sqrt(m)
+    bs = [rng.standard_normal(k * n).astype(np.float32) for _ in range(4)]
+    gys = [rng.standard_normal(m * n).astype(np.float32) for _ in range(4)]
+
+    def program(d):
+        ta, tat = d.new_tensor_by_vector(S([m, k]), a), d.new_tensor_by_vector(S([k, m]), at)
+        tb = [d.new_tensor_by_vector(S([k, n]), b) for b in bs]
+        tgy = [d.new_tensor_by_vector(S([m, n]), g) for g in gys]
+        ga = d.new_tensor_by_constant(S([m, k]), 0)
+        outs = []
+        x = tb[0]
+        for t in range(12):
+            y = d.matmul_fw(ta, tb[t % 4])                     # independent of the chain below
+            gb = d.new_tensor_by_constant(S([k, n]), 0)        # reset per timestep: the pool's block of the last one
+            d.matmul_bw(ta, tb[t % 4], y, tgy[t % 4], ga, gb)  # every call adds into ga
+            y2 = d.matmul_fw(ta, x)                            # a chain: x -> y2 -> x
+            x = d.matmul_fw(tat, y2)
+            if t % 4 == 3:
+                outs += [y.to_vector(), gb.to_vector(), x.to_vector()]
+            del gb, y, y2
+        return outs + [ga.to_vector()]
+
+    lanes, in_order = _run_both(program, storage=storage)
+    _same_bits(lanes, in_order)
+    want = oracle.matmul_fw(a, bs[3], m, k, n, 1, 1)
+    assert norm_rel_err(in_order[0], want) <= 2e-2
