@@ -264,6 +264,21 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
       }
     }
   }
+  // C's old values (an accumulating product) have the longest way to come of everything the epilogue
+  // needs: fetched now, behind the operands' loads, they arrive under the same wait.  (Only the workgroup
+  // that writes a tile touches that part of C in this launch, so the values stay current.)
+  uint16_t *Cz = g.C + (long)z * g.sC;
+  const int g4 = lane >> 4, nl = lane & 15;
+  uint2v old[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + wm * 32 + 16 * i + 4 * g4;
+      const int n = n0 + wn * 32 + 16 * j + nl;
+      old[i][j] = uint2v{0u, 0u};
+      if (g.accumulate && g.vec_c && n < g.N && m + 4 <= g.M) old[i][j] = *reinterpret_cast<const uint2v *>(Cz + m + (long)n * g.ldc);
+    }
   float4v acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -352,8 +367,6 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
   }
 
   // C: block (i, j) holds rows 16 i + 4 (lane / 16) .. + 3 of column 16 j + lane % 16 of the wavefront's 32 x 32
-  uint16_t *Cz = g.C + (long)z * g.sC;
-  const int g4 = lane >> 4, nl = lane & 15;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -363,15 +376,13 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
       if (n >= g.N || m >= g.M) continue;
       uint16_t *p = Cz + m + (long)n * g.ldc;
       if (g.vec_c && m + 4 <= g.M) {
-        uint2v old = {0u, 0u};
-        if (g.accumulate) old = *reinterpret_cast<const uint2v *>(p);
         uint2v out;
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
           float x0 = acc[i][j][2 * w], x1 = acc[i][j][2 * w + 1];
           if (g.accumulate) {
-            x0 += widen<BF16>(old[w] & 0xffffu);
-            x1 += widen<BF16>(old[w] >> 16);
+            x0 += widen<BF16>(old[i][j][w] & 0xffffu);
+            x1 += widen<BF16>(old[i][j][w] >> 16);
           }
           out[w] = narrow<BF16>(x0) | (narrow<BF16>(x1) << 16);
         }
