@@ -56,6 +56,7 @@ set(phip_SRCS
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_conv_pool.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16_big.hip
+  ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_gemm_h16_skinny.hip
   ${PRIMITIV_HIP_BACKEND_DIR}/csrc/phip_matmul.hip
 )
 file(GLOB phip_HDRS "${PRIMITIV_HIP_BACKEND_DIR}/csrc/*.h" "${PRIMITIV_HIP_PHIP_INCLUDE_DIR}/phip.h")

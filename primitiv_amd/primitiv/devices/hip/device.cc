@@ -263,6 +263,10 @@ void HIP::set_overlap(bool on) {
   PHIP_CALL(::phip_set_overlap(ctx_, on ? 1 : 0));
 }
 
+void HIP::set_deferred_zero_fill(bool on) {
+  PHIP_CALL(::phip_set_deferred_zero_fill(ctx_, on ? 1 : 0));
+}
+
 void HIP::dump_description() const {
   char buf[2048];
   PHIP_CALL(::phip_describe(ctx_, buf, sizeof(buf)));

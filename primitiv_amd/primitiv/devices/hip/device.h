@@ -74,6 +74,12 @@ public:
   // stays in the order of its calls.  Off: every launch on one stream.
   void set_overlap(bool on);
 
+  // reset_tensor with the value 0 is only noted, and the gradient operation that
+  // follows writes its result instead of adding it to the zeros (the default):
+  // one launch per gradient of a backward pass instead of two, the same bits.
+  // Off: every fill is launched when it is asked for.
+  void set_deferred_zero_fill(bool on);
+
 private:
   // ---- implemented -------------------------------------------------------
   std::shared_ptr<void> new_handle(const Shape &shape, std::size_t *const allocated_size) override;

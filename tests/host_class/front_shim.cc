@@ -162,6 +162,11 @@ int hc_device_set_overlap(Device *dev, int on) {
   static_cast<primitiv::devices::HIP *>(dev)->set_overlap(on != 0);
   HC_END
 }
+int hc_device_set_deferred_zero_fill(Device *dev, int on) {
+  HC_TRY
+  static_cast<primitiv::devices::HIP *>(dev)->set_deferred_zero_fill(on != 0);
+  HC_END
+}
 int hc_num_devices(U32 *out) {
   HC_TRY
   *out = primitiv::devices::HIP::num_devices();

@@ -63,6 +63,8 @@ def test_device_identity_and_invalid_ids():
     hc.call("hc_device_set_deterministic", d32.ptr, 1)
     hc.call("hc_device_set_overlap", d32.ptr, 0)
     hc.call("hc_device_set_overlap", d32.ptr, 1)
+    hc.call("hc_device_set_deferred_zero_fill", d32.ptr, 0)
+    hc.call("hc_device_set_deferred_zero_fill", d32.ptr, 1)
     p = ctypes.c_void_p()
     hc.call("hc_device_new_hip16", 0, 5, ctypes.byref(p))       # the CUDA16-shaped constructor
     t = ctypes.c_uint32(0)
