@@ -237,6 +237,9 @@ __device__ inline void slab_tile(const LdsArgs &d, unsigned char *lds, uint32_t 
   int sa = 0, sb = 0;  // ring slots of the stage in progress
   auto step = [&](const Frags &cur, Frags &nxt) {
     const int na = next(sa, SA), nb = next(sb, kSlots);
+    // the matrix instructions of a stage go ahead of the other workgroup's loads and bookkeeping on this
+    // compute unit (measured on the output projection: 44.6 -> 43.7 us per timestep)
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int q = 0; q < kMfma; ++q) {
       const int e = q / (2 * MB), i = (q / 2) % MB, j = q & 1;
@@ -250,6 +253,7 @@ __device__ inline void slab_tile(const LdsArgs &d, unsigned char *lds, uint32_t 
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     advance(ca);
     advance(cb);
     // own loads of stage l+2 have landed (later ones may still fly) and own
