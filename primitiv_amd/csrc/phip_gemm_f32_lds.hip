@@ -354,13 +354,14 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   // ---- 64 x 64 tiles
   if (!take) {
     // Measured on M, N in 256 .. 3072, K in 256 .. 1536 against the staged 64 x 64 tiles and the direct
-    // kernel: an overwriting product gains (15 - 35 %) when it is not split and has at least 3/4 tile per
-    // CU (the exchange of partial tiles costs more than the idle CUs); an accumulating product gains
+    // kernel: an overwriting product gains (15 - 35 %) when it is not split and has at least half a tile per
+    // CU (768^3: 32.4 -> 22.4 us; with a quarter, 512^3, the direct kernel is ahead, 13.0 against 15.1 us; the
+    // exchange of partial tiles costs more than the idle CUs); an accumulating product gains
     // (10 - 25 %) from half a tile per CU on, its K cut into ranges of at least 8 tiles until the four
     // places of every CU are filled, the tiles added with atomics.
     side = SBM;
     tiles = tiles_of(SBM);
-    const long least = p.accumulate ? cus / 2 : cus * 3L / 4;
+    const long least = cus / 2;
     if (tiles < least || tiles > 0x7fffffffL || 2L * p.M * p.N * p.batch < tiles * SBM * SBN) return PHIP_OK;
     splits = 1;
     if (p.accumulate && tiles < 4L * cus) {
