@@ -106,8 +106,8 @@ int phip_set_deterministic(phip_ctx *ctx, int on);
  * memory, and every other operation (elementwise work, copies, phip_sync,
  * phip_event_record) waits for both lanes.  The second stream comes into use
  * with the sixth such call in a row and goes out of use with the first
- * operation of another kind that enqueues work; phip_fill_f32 counts as a
- * matmul call here (a backward pass resets every gradient before it adds
+ * operation of another kind that enqueues work; a fill (phip_fill_*) counts
+ * as a matmul call here (a backward pass resets every gradient before it adds
  * products into it).  Products of more than 4 GFLOP and allocation-free calls
  * always run in order.  on == 0 puts every launch back
  * on one stream; the environment variable PHIP_OVERLAP=0 makes that the

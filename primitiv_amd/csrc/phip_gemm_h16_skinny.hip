@@ -18,6 +18,10 @@
 //    ticket, the one that draws a tile's last ticket adds the tiles in order, adds C's old value if
 //    the product accumulates, and rounds once.  No atomics on C (there are none for 16-bit
 //    values), the same bits on every run.
+// Small outputs take a second shape of the same idea: 32 x 32 tiles whose four wavefronts split the K range
+// between them (each holds the whole tile, 8 KiB per K tile, up to 18 K tiles resident) and add their tiles
+// through LDS - four times the workgroups for the same output, and K ranges twice as long before anything
+// has to go through memory.
 // Rows may have any even length: the 16-byte loads need 4-byte alignment only, every load's whole
 // offset is checked against the operand's size (what lies outside reads as zero), and a
 // k-contiguous row that ends inside a 16-byte chunk has the rest of that chunk masked in
@@ -56,6 +60,7 @@ struct SkinnyArgs {
   int total_ktiles;  // ktiles_per_r * rbatch
   int accumulate;
   int vec_c;         // C may be moved 8 bytes (4 rows of a column) at a time
+  int small;         // 32 x 32 tiles with the wavefronts splitting K (skinny_tile_small) instead of 64 x 64
   uint32_t a_bytes, b_bytes;  // bytes of one sample of each operand
   float *partial;    // splits > 1: 64 x 64 fp32 tiles, ((z * tiles + tile) * splits + split) * 4096 floats each
   uint32_t *tickets; // splits > 1: one zeroed counter per output tile, left zeroed
@@ -400,11 +405,237 @@ __device__ inline void skinny_tile(const SkinnyArgs &g, unsigned char *lds, uint
     }
 }
 
+// ---- 32 x 32 tiles, the wavefronts split K ---------------------------------------------------------------
+
+constexpr int SM = 32, SN = 32;
+constexpr int kRegionS = 32 * BK * 2;  // bytes of one operand's K tile: 32 rows (m or n) x 64 k
+constexpr int kStageS = 2 * kRegionS;
+constexpr int kMaxStagesS = 18;        // 144 KiB
+constexpr int kReduceBytesS = 16384;   // the four wavefronts' tiles, when they are added up
+
+// One piece (16 bytes per lane) of each of eight partial tiles, all in flight at once, and the wait.
+__device__ inline void load_eight_device_scope(float4v (&v)[8], const float *const (&q)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n\t"
+      "global_load_dwordx4 %1, %9, off sc1\n\t"
+      "global_load_dwordx4 %2, %10, off sc1\n\t"
+      "global_load_dwordx4 %3, %11, off sc1\n\t"
+      "global_load_dwordx4 %4, %12, off sc1\n\t"
+      "global_load_dwordx4 %5, %13, off sc1\n\t"
+      "global_load_dwordx4 %6, %14, off sc1\n\t"
+      "global_load_dwordx4 %7, %15, off sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+      : "v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]), "v"(q[4]), "v"(q[5]), "v"(q[6]), "v"(q[7])
+      : "memory");
+}
+
+// A wavefront's one load instruction per operand and K tile (the four wavefronts fill the 4 KiB region).
+//  * k-contiguous operand: 32 rows of 128 bytes, chunk c of row x at position c ^ ((x >> 1) & 7);
+//  * m/n-contiguous operand: 64 rows (k) of 32 elements = 4 chunks; chunk c of row k at position
+//    c ^ (((k >> 1) & 1) << 1): the four k rows of a transposing read land in different banks.
+template <bool KMAJOR>
+struct LoaderS {
+  uint32_t off;
+  int kpos;
+  uint32_t step;
+
+  __device__ inline void init(long ld, int x0, int X, int wave, int lane) {
+    if constexpr (KMAJOR) {
+      const int x = wave * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((x >> 1) & 7);
+      off = x0 + x < X ? (uint32_t)(((long)(x0 + x) * ld + c * 8) * 2) : kOutOfRange;
+      kpos = c * 8;
+    } else {
+      const int k = wave * 16 + (lane >> 2);
+      const int c = (lane & 3) ^ (((k >> 1) & 1) << 1);
+      off = x0 + c * 8 < X ? (uint32_t)(((long)k * ld + x0 + c * 8) * 2) : kOutOfRange;
+      kpos = k;
+    }
+    step = KMAJOR ? (uint32_t)(BK * 2) : (uint32_t)(BK * ld * 2);
+  }
+
+  __device__ inline void issue(uint4v rsrc, uint32_t lds_region, int wave, int kin, int K) const {
+    const bool inside = kin * BK + kpos < K;
+    const uint32_t v = inside ? off + (uint32_t)kin * step : kOutOfRange;
+    lds_dma_b128(rsrc, lds_region + (uint32_t)(wave * 1024), v | (off & kOutOfRange));
+  }
+};
+
+template <bool KMAJOR>
+__device__ inline uint4v read_fragment_small(uint32_t region, int xb, int t, int lane) {
+  if constexpr (KMAJOR) {
+    return read_fragment<true>(region, xb, t, lane);  // the same image: rows of 128 bytes
+  } else {
+    const int g = lane >> 4, cc = (lane & 15) >> 2, a = lane & 3;
+    const uint32_t p = region + (uint32_t)((32 * t + 8 * g + cc) * 64 + (((xb / 8 + (a >> 1)) ^ (((cc >> 1) & 1) << 1)) * 16) + (a & 1) * 8);
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(lds_ptr<short4v>(p));
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(lds_ptr<short4v>(p + 4 * 64));
+    uint4v r;
+    r.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+    r.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+    r.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+    r.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+    return r;
+  }
+}
+
+// One workgroup's work on a 32 x 32 tile.  `lds` holds max(stages x kStageS, kReduceBytesS) bytes.
 template <bool A_KMAJOR, bool B_KMAJOR, bool BF16>
-__global__ __launch_bounds__(kThreads) void gemm_h16_skinny_kernel(const SkinnyArgs g) {
+__device__ inline void skinny_tile_small(const SkinnyArgs &g, unsigned char *lds, uint32_t *flag, int bid, int nblk) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  int t = xcd_remap(bid, nblk);
+  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
+  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
+  const int split = t % g.splits;
+  const int z = t / g.splits;
+  const int m0 = tile_m * SM, n0 = tile_n * SN;
+
+  const int kb = (int)((long)split * g.total_ktiles / g.splits);
+  const int ke = (int)((long)(split + 1) * g.total_ktiles / g.splits);
+  const int n_st = ke - kb;
+
+  LoaderS<A_KMAJOR> la;
+  LoaderS<B_KMAJOR> lb;
+  la.init(g.lda, m0, g.M, wave, lane);
+  lb.init(g.ldb, n0, g.N, wave, lane);
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
+  const uint16_t *Az = g.A + (long)z * g.sA;
+  const uint16_t *Bz = g.B + (long)z * g.sB;
+  {
+    int r = kb / g.ktiles_per_r, kin = kb - r * g.ktiles_per_r;
+    for (int s = 0; s < n_st; ++s) {
+      const uint4v ra = make_rsrc_words(Az + (long)r * g.rA, g.a_bytes);
+      const uint4v rb = make_rsrc_words(Bz + (long)r * g.rB, g.b_bytes);
+      const uint32_t stage = lds_base + (uint32_t)s * kStageS;
+      la.issue(ra, stage, wave, kin, g.K);
+      lb.issue(rb, stage + kRegionS, wave, kin, g.K);
+      if (++kin == g.ktiles_per_r) {
+        kin = 0;
+        ++r;
+      }
+    }
+  }
+  // after the sum over the wavefronts, wavefront w owns the 16 x 16 block (w / 2, w % 2) of the tile
+  uint16_t *Cz = g.C + (long)z * g.sC;
+  const int g4 = lane >> 4, nl = lane & 15;
+  const int m = m0 + 16 * (wave >> 1) + 4 * g4;
+  const int n = n0 + 16 * (wave & 1) + nl;
+  uint2v old = {0u, 0u};
+  if (g.accumulate && g.vec_c && n < g.N && m + 4 <= g.M) old = *reinterpret_cast<const uint2v *>(Cz + m + (long)n * g.ldc);
+  float4v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  {
+    // k steps of 32: wavefront w takes steps w, w + 4, ... of the workgroup's range
+    const bool ragged = (A_KMAJOR || B_KMAJOR) && (g.K & 7) != 0;
+    const int kin0 = kb % g.ktiles_per_r;
+    for (int ks = wave; ks < 2 * n_st; ks += 4) {
+      const int s = ks >> 1, tt = ks & 1;
+      const uint32_t stage = lds_base + (uint32_t)s * kStageS;
+      const int kin = (kin0 + s) % g.ktiles_per_r;
+      uint4v fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = read_fragment_small<A_KMAJOR>(stage, 16 * i, tt, lane);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = read_fragment_small<B_KMAJOR>(stage + kRegionS, 16 * j, tt, lane);
+      if (ragged && kin == g.ktiles_per_r - 1) {
+        int valid = g.K - (kin * BK + 32 * tt + 8 * (lane >> 4));
+        valid = valid < 0 ? 0 : (valid > 8 ? 8 : valid);
+        if constexpr (A_KMAJOR) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) fa[i] = keep_first(fa[i], valid);
+        }
+        if constexpr (B_KMAJOR) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) fb[j] = keep_first(fb[j], valid);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma<BF16>(fa[i], fb[j], acc[i][j]);
+    }
+  }
+  // the four wavefronts' tiles, added in the order of the wavefronts: wavefront w sums block w
+  __syncthreads();  // every wavefront is done with the operands in LDS
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) *lds_ptr<float4v>(lds_base + (uint32_t)(((wave * 4 + 2 * i + j) * 64 + lane) * 16)) = acc[i][j];
+  __syncthreads();
+  float4v blk = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) blk += *lds_ptr<const float4v>(lds_base + (uint32_t)(((w * 4 + wave) * 64 + lane) * 16));
+
+  if (g.splits > 1) {
+    const long tile_id = ((long)z * g.tiles_n + tile_n) * g.tiles_m + tile_m;
+    float *P = g.partial + (tile_id * g.splits + split) * (long)(SM * SN) + wave * 256 + lane * 4;
+    store_device_scope(P, blk);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      const uint32_t ticket = __hip_atomic_fetch_add(g.tickets + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = ticket == (uint32_t)g.splits - 1u;
+      if (last) __hip_atomic_store(g.tickets + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (*flag == 0) return;
+    const float *Q = g.partial + tile_id * g.splits * (long)(SM * SN) + wave * 256 + lane * 4;
+    blk = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int r0 = 0; r0 < g.splits; r0 += 8) {
+      float4v part[8];
+      const float *q[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) q[u] = Q + (long)(r0 + u < g.splits ? r0 + u : r0) * (SM * SN);
+      load_eight_device_scope(part, q);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (r0 + u < g.splits) blk += part[u];
+    }
+  }
+
+  if (n >= g.N || m >= g.M) return;
+  uint16_t *p = Cz + m + (long)n * g.ldc;
+  if (g.vec_c && m + 4 <= g.M) {
+    uint2v out;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      float x0 = blk[2 * w], x1 = blk[2 * w + 1];
+      if (g.accumulate) {
+        x0 += widen<BF16>(old[w] & 0xffffu);
+        x1 += widen<BF16>(old[w] >> 16);
+      }
+      out[w] = narrow<BF16>(x0) | (narrow<BF16>(x1) << 16);
+    }
+    *reinterpret_cast<uint2v *>(p) = out;
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      if (m + v < g.M) {
+        float x = blk[v];
+        if (g.accumulate) x += widen<BF16>(p[v]);
+        p[v] = (uint16_t)narrow<BF16>(x);
+      }
+    }
+  }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, bool BF16>
+__global__ __launch_bounds__(kThreads, 4) void gemm_h16_skinny_kernel(const SkinnyArgs g) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_skinny[];
   __shared__ uint32_t flag;
-  skinny_tile<A_KMAJOR, B_KMAJOR, BF16>(g, lds_skinny, &flag, blockIdx.x, gridDim.x);
+  if (g.small) skinny_tile_small<A_KMAJOR, B_KMAJOR, BF16>(g, lds_skinny, &flag, blockIdx.x, gridDim.x);
+  else skinny_tile<A_KMAJOR, B_KMAJOR, BF16>(g, lds_skinny, &flag, blockIdx.x, gridDim.x);
 }
 
 // Both gradient products of one matmul_bw call in one grid: workgroups below `first` run ga += gy . b^T
@@ -413,13 +644,18 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_skinny_kernel(const SkinnyA
 // The second problem's workgroups start at `second_at`, a multiple of 8, so that both problems meet the XCDs
 // in the order their tile numbering expects; workgroups between the two do nothing.
 template <bool BF16>
-__global__ __launch_bounds__(kThreads) void gemm_h16_skinny_pair_kernel(const SkinnyArgs g1, const SkinnyArgs g2, int first,
+__global__ __launch_bounds__(kThreads, 4) void gemm_h16_skinny_pair_kernel(const SkinnyArgs g1, const SkinnyArgs g2, int first,
                                                                          int second_at) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_skinny[];
   __shared__ uint32_t flag;
   const int bid = blockIdx.x;
-  if (bid < first) skinny_tile<false, false, BF16>(g1, lds_skinny, &flag, bid, first);
-  else if (bid >= second_at) skinny_tile<true, true, BF16>(g2, lds_skinny, &flag, bid - second_at, (int)gridDim.x - second_at);
+  if (bid < first) {
+    if (g1.small) skinny_tile_small<false, false, BF16>(g1, lds_skinny, &flag, bid, first);
+    else skinny_tile<false, false, BF16>(g1, lds_skinny, &flag, bid, first);
+  } else if (bid >= second_at) {
+    if (g2.small) skinny_tile_small<true, true, BF16>(g2, lds_skinny, &flag, bid - second_at, (int)gridDim.x - second_at);
+    else skinny_tile<true, true, BF16>(g2, lds_skinny, &flag, bid - second_at, (int)gridDim.x - second_at);
+  }
 }
 
 struct SkinnyPlan {
@@ -427,6 +663,8 @@ struct SkinnyPlan {
   long tiles;   // output tiles times samples
   long grid;    // tiles times K ranges
   int stages;   // K tiles of the longest range
+  int lds;      // bytes of LDS a workgroup needs
+  int tile_floats;  // elements of one output tile (one partial tile of a split product)
 };
 
 // False when the problem is not one for this kernel.  `places_per_cu` caps how many workgroups may share a
@@ -447,39 +685,52 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
   const int cus = ctx->prop.multiProcessorCount;
   const int ktiles_per_r = (p.K + BK - 1) / BK;
   const long total_ktiles = (long)ktiles_per_r * p.rbatch;
-  const long tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TN - 1) / TN;
-  const long tiles = tiles_m * tiles_n * p.batch;
-  if (total_ktiles > 100000 || tiles > kTicketSlots) return false;
+  if (total_ktiles > 100000) return false;
 
-  // Stages per workgroup: the choice that a small cost model likes best (microseconds): the loads of the
-  // workgroups that share a compute unit (about 0.4 per 16 KiB K tile), the exchange of partial tiles when
-  // K is cut (store, ticket, then one round trip through memory per four ranges), and a second round of
-  // workgroups if the grid does not fit the chip at once.
-  int best_s = 0;
+  // Tile shape and stages per workgroup: the choice that a small cost model likes best (microseconds): the
+  // loads of the workgroups that share a compute unit (about 0.4 per 16 KiB), the exchange of partial tiles
+  // when K is cut (store, ticket, then one round trip through memory per four - small tiles: eight - ranges),
+  // the sum over the wavefronts of a small tile, and a second round of workgroups if the grid does not fit
+  // the chip at once.  Ties go to the large tiles, which load each operand fewer times.
+  int best_s = 0, best_small = 0;
+  long best_tiles = 0;
   double best = 0.0;
-  for (int s = 1; s <= kMaxStages; ++s) {
-    const long splits = (total_ktiles + s - 1) / s;
-    const int s_eff = (int)((total_ktiles + splits - 1) / splits);
-    if (s_eff != s && s != kMaxStages) continue;  // the same cut as a smaller s
-    int occ = (160 * 1024) / (s_eff * kStage);
-    if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
-    if (places_per_cu > 0 && occ > places_per_cu) occ = places_per_cu;
-    if (occ < 1) continue;
-    const long grid = tiles * splits;
-    if (grid > 0x7fffffffL) continue;
-    if (splits > 1 && (size_t)grid * TM * TN * 4 > ((size_t)64 << 20)) continue;
-    const long places = (long)cus * occ;
-    const long rounds = (grid + places - 1) / places;
-    long per_cu = (grid + cus - 1) / cus;
-    if (per_cu > occ) per_cu = occ;
-    const double cost = rounds * (1.0 + 0.4 * s_eff * per_cu) + (splits > 1 ? 2.0 + 1.2 * ((splits + 3) / 4) : 0.0);
-    if (best_s == 0 || cost < best) {
-      best = cost;
-      best_s = s_eff;
+  for (int small = 0; small < 2; ++small) {
+    const int side = small ? SM : TM, stage_bytes = small ? kStageS : kStage, max_s = small ? kMaxStagesS : kMaxStages;
+    const long tiles = (long)((p.M + side - 1) / side) * ((p.N + side - 1) / side) * p.batch;
+    if (tiles > kTicketSlots) continue;
+    for (int s = 1; s <= max_s; ++s) {
+      const long splits = (total_ktiles + s - 1) / s;
+      const int s_eff = (int)((total_ktiles + splits - 1) / splits);
+      if (s_eff != s && s != max_s) continue;  // the same cut as a smaller s
+      int lds = s_eff * stage_bytes;
+      if (small && lds < kReduceBytesS) lds = kReduceBytesS;
+      int occ = (160 * 1024) / lds;
+      if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
+      if (places_per_cu > 0 && occ > places_per_cu) occ = places_per_cu;
+      if (occ < 1) continue;
+      const long grid = tiles * splits;
+      if (grid > 0x7fffffffL) continue;
+      if (splits > 1 && (size_t)grid * side * side * 4 > ((size_t)64 << 20)) continue;
+      const long places = (long)cus * occ;
+      const long rounds = (grid + places - 1) / places;
+      long per_cu = (grid + cus - 1) / cus;
+      if (per_cu > occ) per_cu = occ;
+      const double loads = 0.4 * s_eff * per_cu * stage_bytes / kStage;
+      const double exchange = splits > 1 ? 2.0 + 1.2 * ((splits + (small ? 7 : 3)) / (small ? 8 : 4)) : 0.0;
+      const double cost = rounds * (1.0 + (small ? 0.3 : 0.0) + loads) + exchange;
+      if (best_s == 0 || cost < best - 1e-9) {
+        best = cost;
+        best_s = s_eff;
+        best_small = small;
+        best_tiles = tiles;
+      }
     }
   }
   if (best_s == 0) return false;
   const long splits = (total_ktiles + best_s - 1) / best_s;
+  const int side = best_small ? SM : TM;
+  const long tiles = best_tiles;
 
   SkinnyArgs &a = plan->a;
   a.A = static_cast<const uint16_t *>(p.A);
@@ -489,13 +740,14 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
   a.lda = p.lda; a.ldb = p.ldb; a.ldc = p.ldc;
   a.sA = p.sA; a.sB = p.sB; a.sC = p.sC;
   a.rA = p.rA; a.rB = p.rB;
-  a.tiles_m = (int)tiles_m;
-  a.tiles_n = (int)tiles_n;
+  a.tiles_m = (p.M + side - 1) / side;
+  a.tiles_n = (p.N + side - 1) / side;
   a.splits = (int)splits;
   a.ktiles_per_r = ktiles_per_r;
   a.total_ktiles = (int)total_ktiles;
   a.accumulate = p.accumulate ? 1 : 0;
   a.vec_c = reinterpret_cast<uintptr_t>(p.C) % 8 == 0 && p.ldc % 4 == 0 && p.sC % 4 == 0;
+  a.small = best_small;
   a.a_bytes = (uint32_t)a_bytes;
   a.b_bytes = (uint32_t)b_bytes;
   a.partial = nullptr;
@@ -503,6 +755,9 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
   plan->tiles = tiles;
   plan->grid = tiles * splits;
   plan->stages = (int)((total_ktiles + splits - 1) / splits);
+  plan->lds = plan->stages * (best_small ? kStageS : kStage);
+  if (best_small && plan->lds < kReduceBytesS) plan->lds = kReduceBytesS;
+  plan->tile_floats = side * side;
   return true;
 }
 
@@ -511,7 +766,7 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
 int prepare_exchange(phip_ctx *ctx, SkinnyPlan *plan, void **block) {
   *block = nullptr;
   if (plan->a.splits <= 1) return PHIP_OK;
-  const int rc = scratch_alloc(ctx, (size_t)plan->grid * TM * TN * sizeof(float), block);
+  const int rc = scratch_alloc(ctx, (size_t)plan->grid * plan->tile_floats * sizeof(float), block);
   if (rc != PHIP_OK) return rc;
   plan->a.partial = static_cast<float *>(*block);
   plan->a.tickets = tile_tickets(ctx);
@@ -534,7 +789,7 @@ int gemm_h16_skinny(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   void *block = nullptr;
   int rc = prepare_exchange(ctx, &plan, &block);
   if (rc != PHIP_OK) return rc;
-  const int lds = plan.stages * kStage;
+  const int lds = plan.lds;
   const bool bf = elem == Elem::BF16;
 #define PHIP_SKINNY(SLOT, AK, BKM)                                                                                 \
   do {                                                                                                             \
@@ -555,7 +810,7 @@ int gemm_h16_skinny(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   if (block) scratch_free(ctx, block);  // the stream is in order: reusable behind this launch
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
-  note_kernel(ctx, "h16_skinny");
+  note_kernel(ctx, plan.a.small ? "h16_skinny32" : "h16_skinny");
   *handled = true;
   return PHIP_OK;
 }
@@ -568,9 +823,9 @@ int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, E
   SkinnyPlan p1, p2;
   // both grids resident at once: each problem is planned for half of the places
   if (!plan_skinny(ctx, first, &p1, 4) || !plan_skinny(ctx, second, &p2, 4)) return PHIP_OK;
-  const int stages = p1.stages > p2.stages ? p1.stages : p2.stages;
+  const int lds = p1.lds > p2.lds ? p1.lds : p2.lds;
   const int cus = ctx->prop.multiProcessorCount;
-  int occ = (160 * 1024) / (stages * kStage);
+  int occ = (160 * 1024) / lds;
   if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
   const long second_at = (p1.grid + 7) / 8 * 8;
   if (second_at + p2.grid > (long)cus * occ) return PHIP_OK;  // would take a second round: two launches do as well
@@ -583,7 +838,6 @@ int gemm_h16_skinny_pair(phip_ctx *ctx, const Gemm &first, const Gemm &second, E
     else p2.a.tickets = tile_tickets(ctx) + p1.tiles;
   }
   if (rc == PHIP_OK) {
-    const int lds = stages * kStage;
     const unsigned grid = (unsigned)(second_at + p2.grid);
     if (elem == Elem::BF16) {
       auto kern = gemm_h16_skinny_pair_kernel<true>;
