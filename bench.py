@@ -37,11 +37,13 @@ STORAGE_CODE = {"f32": 0, "f16": 1, "bf16": 2}
 # y += x of known size in the same runs), summed over a step's launches ("HBM bytes per step by the
 # counters" there).  Algorithmic bytes for comparison are Workload.bytes_per_step().
 COUNTER_TRAFFIC_BYTES_PER_STEP = {
-    "square_batched": 762.4e6,       # 206.14 + 283.93 + 272.32 MB: the three gemm_f32_lds_kernel launches
+    "square_batched": 762.6e6,       # 206.23 + 284.09 + 272.26 MB: the three gemm_f32_lds_kernel launches
     "dense": 14.58e6,                # gemm_f32_tile16_kernel 7.06 + gemm_f32_pair_kernel 7.52 MB
-    "rnn_gate": 872.4e6,             # 30 x (9.64 + 19.44 MB)
-    "output_projection": 4473.4e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.16 MB)
-    "half_storage": 6273.2e6,        # 2 x 2122.67 + 1960.7 + 67.17 MB (transposed copy of a)
+    "rnn_gate": 873.0e6,             # 30 x (9.64 + 19.47 MB)
+    "output_projection": 4468.9e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.03 MB)
+    "half_storage": 6284.7e6,        # 2 x 2122.68 + 1972.15 + 67.17 MB (transposed copy of a)
+    "rnn_gate:f16": 486.9e6,         # 30 x (gemm_h16_skinny_kernel 4.83 + gemm_h16_skinny_pair_kernel 11.40 MB)
+    "output_projection:f16": 3150.3e6,  # 35 x (30.44 + 36.69 + 22.88 MB: three gemm_h16_skinny_kernel launches)
 }
 # per launch of the headline kernel (average of its three operand-layout instantiations)
 HEADLINE_TRAFFIC_BYTES = COUNTER_TRAFFIC_BYTES_PER_STEP["square_batched"] / 3
@@ -273,14 +275,6 @@ def _workload(name):
     return WORKLOADS[name]
 
 
-# Kernel launches per matmul_fw + matmul_bw call pair as the library plans them today (the kernel
-# traces in profiles/): one forward launch and both gradients in one launch for the three
-# per-timestep fp32 workloads, three launches for the batched squares, a transposed copy of `a` plus
-# three products for the 16-bit workload; anything else: three.
-LAUNCHES_PER_CALL_PAIR = {"dense": 2, "rnn_gate": 2, "output_projection": 2, "square_batched": 3,
-                          "half_storage": 4, "half_storage:bf16": 4}
-
-
 def _figures(w, per_step_s):
     tflops = w.flops_per_step() * w.steps / per_step_s / 1e12
     gbs = w.bytes_per_step() * w.steps / per_step_s / 1e9
@@ -301,7 +295,8 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False, 
     loops = Loops(dev, res)
     dev.gemm_trace(True)
     loops.raw(1, 0)
-    kernels = dev.gemm_trace(False)[:8]
+    trace = dev.gemm_trace(False)      # every kernel that the step's matmul calls launched, helpers included
+    kernels = trace[:8]
     warm_steps, warm_s = loops.settle(warmup)
     ms, host_ms = loops.raw(steps, 0)                       # the step of record: a C++ caller's loop
     out = {"workload": name, "dtype": w.storage, "calls_per_step": w.steps, "steps_timed": steps,
@@ -309,7 +304,7 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False, 
            "ms_per_step": ms, "ms_per_step_host_clock": host_ms,
            "streams": "one" if not lanes_for_record else "library default (two lanes for runs of independent products)",
            "gemm_kernels_first_timestep": kernels}
-    launches = LAUNCHES_PER_CALL_PAIR.get(name, 3) * w.steps
+    launches = len(trace)
     out["kernel_launches_per_step"] = launches
     out["us_per_kernel_launch"] = ms * 1e3 / launches
     out.update(_figures(w, ms * 1e-3))

@@ -236,6 +236,7 @@ inline int zero_c(phip_ctx *ctx, const Gemm &p) {
   hipLaunchKernelGGL(zero_c_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream, static_cast<float *>(p.C),
                      p.M, p.N, p.ldc, p.sC, p.batch);
   PHIP_LAUNCH_CHECK();
+  note_kernel(ctx, "zero_c");
   return PHIP_OK;
 }
 

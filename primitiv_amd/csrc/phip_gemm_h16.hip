@@ -442,6 +442,7 @@ int launch_tile_h(phip_ctx *ctx, const Gemm &p, GemmArgsH a, bool vec_a, bool ve
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((finish_split_h16_kernel<BF16>), dim3((unsigned)blocks), dim3(kThreads), 0, ctx->stream,
                        a.partial, a.C, p.M, p.N, p.ldc, p.sC, p.batch, (int)splits, a.accumulate);
+    note_kernel(ctx, "h16_finish_split");
     scratch_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
   }
   PHIP_LAUNCH_CHECK();

@@ -103,6 +103,7 @@ static int matmul_fw(phip_ctx *ctx, Elem elem, const void *a, const void *b, voi
     rc = elem == Elem::F16 ? phip_transpose_fw_f16(ctx, a, at.ptr, di, dj, 1)
                            : phip_transpose_fw_bf16(ctx, a, at.ptr, di, dj, 1);
     if (rc != PHIP_OK) return rc;
+    note_kernel(ctx, "transposed_copy");
     g.A = at.ptr;      // a^T: element (m, k) at k + m*dj
     g.lda = dj;
     g.a_kmajor = true;

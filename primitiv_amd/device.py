@@ -429,7 +429,7 @@ class HIP:
     def gemm_trace(self, on=True):
         """Names of the GEMM kernels that this device's matmul calls went to since the previous call
         (a list, launch order per stream); `on` switches the note-taking on or off from here on."""
-        buf = ctypes.create_string_buffer(4096)
+        buf = ctypes.create_string_buffer(1 << 16)
         _lib.call("phip_gemm_trace", self._ctx, 1 if on else 0, buf, len(buf))
         return buf.value.decode().split()
 
