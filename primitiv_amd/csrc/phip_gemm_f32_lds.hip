@@ -22,8 +22,99 @@ constexpr int kRegion = 16384;            // bytes per operand per stage
 constexpr int kStage = 2 * kRegion;
 constexpr int kLdsBytes = 2 * kStage;
 
-template <bool A_KMAJOR, bool B_KMAJOR, bool SPLIT>
+// Which output tile and which K range a workgroup takes.
+//  * unsplit: one tile each, the whole K range;
+//  * split: every tile is shared by `splits` workgroups;
+//  * mixed (whole_tiles > 0): the tiles do not fill a whole number of rounds on the chip.  The first
+//    `whole_tiles` workgroups (a multiple of the CU count) take one tile each; the tiles that are left - too
+//    few for a round of their own, so that a few CUs would carry one tile more than the others - are cut
+//    into `splits` K ranges each, whose workgroups spread over all CUs behind the whole tiles.
+struct TileWork {
+  int tile_m, tile_n, z;
+  int split;    // K range of a shared tile
+  bool shared;  // the tile is shared: meet through atomics or partial tiles
+  int tail;     // mixed: index of the shared tile among the shared ones
+};
+
+template <int MODE>
+__device__ inline TileWork tile_work(const LdsArgs &d) {
+  constexpr bool SPLIT = MODE != 0;
+  const GemmArgs &g = d.g;
+  TileWork w;
+  w.split = 0;
+  w.shared = SPLIT;
+  w.tail = 0;
+  int t;
+  if constexpr (MODE == 2) {
+    const int bid = blockIdx.x;
+    if (bid < d.whole_tiles) {
+      t = xcd_remap(bid, d.whole_tiles);
+      w.shared = false;
+    } else {
+      const int rest = (int)gridDim.x - d.whole_tiles;
+      const int tails = rest / g.splits;
+      const int u = xcd_remap(bid - d.whole_tiles, rest);
+      w.tail = u % tails;
+      w.split = u / tails;
+      t = d.whole_tiles + w.tail;
+    }
+    w.tile_m = t % g.tiles_m; t /= g.tiles_m;
+    w.tile_n = t % g.tiles_n; t /= g.tiles_n;
+    w.z = t;
+    return w;
+  } else {
+  t = xcd_remap(blockIdx.x, gridDim.x);
+  w.tile_m = t % g.tiles_m; t /= g.tiles_m;
+  w.tile_n = t % g.tiles_n; t /= g.tiles_n;
+  if (SPLIT) {
+    w.split = t % g.splits;
+    t /= g.splits;
+  }
+  w.z = t;
+  return w;
+  }
+}
+
+// Partial tiles of a mixed launch: SIDE x SIDE floats per shared tile and K range, tile-local coordinates
+// (elements outside the matrix are zeros: their operands were zero-filled by the loads).  Same device-scope
+// accesses and ticket as store_partial / sum_partials / last_of_tile.
+template <int NV, int SIDE>
+__device__ inline void store_tile_partial(float *P, int row0, int col0, int lane, const int (&nq)[NV], const float (&vals)[NV]) {
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+#pragma unroll
+  for (int q = 0; q < NV; ++q)
+    __hip_atomic_store(P + m + (ncol + nq[q]) * SIDE, vals[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int NV, int SIDE>
+__device__ inline void sum_tile_partials(const float *P, int splits, int row0, int col0, int lane, const int (&nq)[NV],
+                                         float (&vals)[NV]) {
+  const int m = row0 + (lane & 31);
+  const int ncol = col0 + 4 * (lane >> 5);
+  constexpr int kPer = SIDE * SIDE;
+#pragma unroll
+  for (int q = 0; q < NV; ++q) vals[q] = 0.0f;
+  for (int r0 = 0; r0 < splits; r0 += 4) {
+    float part[4][NV];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int q = 0; q < NV; ++q)
+        part[u][q] = __hip_atomic_load(P + (r0 + u < splits ? r0 + u : r0) * kPer + m + (ncol + nq[q]) * SIDE,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int q = 0; q < NV; ++q)
+        if (r0 + u < splits) vals[q] += part[u][q];
+  }
+}
+
+// MODE 0: unsplit, 1: every tile shared by K ranges, 2: mixed (see TileWork).
+template <bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs d) {
+  constexpr bool SPLIT = MODE != 0;
   const GemmArgs &g = d.g;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
@@ -32,15 +123,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
 
-  int t = xcd_remap(blockIdx.x, gridDim.x);
-  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
-  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
-  int split = 0;
-  if constexpr (SPLIT) {
-    split = t % g.splits;
-    t /= g.splits;
-  }
-  const int z = t;
+  const TileWork tw = tile_work<MODE>(d);
+  const int tile_m = tw.tile_m, tile_n = tw.tile_n, z = tw.z, split = tw.split;
   const int m0 = tile_m * LBM, n0 = tile_n * LBN;
 
   DmaLoader<A_KMAJOR> la;
@@ -64,8 +148,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   // K tiles [kt_base, kt_base + kt_end) belong to this workgroup
-  const int kt_base = SPLIT ? (int)((long)split * g.total_ktiles / g.splits) : 0;
-  const int kt_end = SPLIT ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
+  const int kt_base = tw.shared ? (int)((long)split * g.total_ktiles / g.splits) : 0;
+  const int kt_end = tw.shared ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
   auto issue_tile = [&](int kt, int q) {
     // instruction q of the 8 that move K tile kt (4 for A, then 4 for B)
@@ -128,7 +212,34 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
   int ns[16];
 #pragma unroll
   for (int v = 0; v < 16; ++v) ns[v] = 8 * (v / 4) + (v % 4);
-  if constexpr (SPLIT) {
+  if constexpr (MODE == 2) {
+    if (tw.shared && g.atomic == 2) {
+      // mixed launch: tile-sized partial tiles of the shared tiles only
+      __shared__ uint32_t last_flag_mixed;
+      float *P = g.partial + (long)tw.tail * g.splits * (LBM * LBN);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float vals[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) vals[v] = acc[i][j][v];
+          store_tile_partial<16, LBM>(P + split * (LBM * LBN), wm * 64 + i * 32, wn * 64 + j * 32, lane, ns, vals);
+        }
+      if (!last_of_tile(g, tw.tail, &last_flag_mixed)) return;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float vals[16];
+          sum_tile_partials<16, LBM>(P, g.splits, wm * 64 + i * 32, wn * 64 + j * 32, lane, ns, vals);
+          emit_c<16>(Cz, g.ldc, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, g.M, g.N, interior, ns, vals, 0,
+                     g.accumulate);
+        }
+      return;
+    }
+  }
+  if constexpr (MODE == 1) {
     if (g.atomic == 2) {
       // leave the partial tile; the last workgroup of the output tile adds the ranges in order
       __shared__ uint32_t last_flag;
@@ -162,7 +273,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs
 #pragma unroll
       for (int v = 0; v < 16; ++v) vals[v] = acc[i][j][v];
       emit_c<16>(Cz, g.ldc, m0 + wm * 64 + i * 32, n0 + wn * 64 + j * 32, lane, g.M, g.N, interior, ns, vals,
-                 SPLIT ? g.atomic : 0, g.accumulate);
+                 tw.shared ? g.atomic : 0, g.accumulate);
     }
 }
 
@@ -175,8 +286,9 @@ constexpr int kRegion64 = 8192;
 constexpr int kStage64 = 2 * kRegion64;
 constexpr int kLds64Bytes = 2 * kStage64;
 
-template <bool A_KMAJOR, bool B_KMAJOR, bool SPLIT>
+template <bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsArgs d) {
+  constexpr bool SPLIT = MODE != 0;
   const GemmArgs &g = d.g;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
@@ -185,15 +297,8 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
 
-  int t = xcd_remap(blockIdx.x, gridDim.x);
-  const int tile_m = t % g.tiles_m; t /= g.tiles_m;
-  const int tile_n = t % g.tiles_n; t /= g.tiles_n;
-  int split = 0;
-  if constexpr (SPLIT) {
-    split = t % g.splits;
-    t /= g.splits;
-  }
-  const int z = t;
+  const TileWork tw = tile_work<MODE>(d);
+  const int tile_m = tw.tile_m, tile_n = tw.tile_n, z = tw.z, split = tw.split;
   const int m0 = tile_m * SBM, n0 = tile_n * SBN;
 
   DmaLoader<A_KMAJOR, SBM> la;
@@ -213,8 +318,8 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 
   // K tiles [kt_base, kt_base + kt_end) belong to this workgroup
-  const int kt_base = SPLIT ? (int)((long)split * g.total_ktiles / g.splits) : 0;
-  const int kt_end = SPLIT ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
+  const int kt_base = tw.shared ? (int)((long)split * g.total_ktiles / g.splits) : 0;
+  const int kt_end = tw.shared ? (int)((long)(split + 1) * g.total_ktiles / g.splits) - kt_base : g.total_ktiles;
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
   auto issue_tile = [&](int kt, int q) {
     // instruction q of the 4 that move K tile kt (2 for A, then 2 for B)
@@ -279,7 +384,18 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
     ns[v] = 8 * (v / 4) + (v % 4);
     vals[v] = acc[v];
   }
-  if constexpr (SPLIT) {
+  if constexpr (MODE == 2) {
+    if (tw.shared && g.atomic == 2) {
+      __shared__ uint32_t last_flag_mixed;
+      float *P = g.partial + (long)tw.tail * g.splits * (SBM * SBN);
+      store_tile_partial<16, SBM>(P + split * (SBM * SBN), wm * 32, wn * 32, lane, ns, vals);
+      if (!last_of_tile(g, tw.tail, &last_flag_mixed)) return;
+      sum_tile_partials<16, SBM>(P, g.splits, wm * 32, wn * 32, lane, ns, vals);
+      emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, 0, g.accumulate);
+      return;
+    }
+  }
+  if constexpr (MODE == 1) {
     if (g.atomic == 2) {
       __shared__ uint32_t last_flag;
       store_partial<16>(g, z, split, row0, col0, lane, ns, vals);
@@ -289,7 +405,7 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
       return;
     }
   }
-  emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, SPLIT ? g.atomic : 0, g.accumulate);
+  emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, tw.shared ? g.atomic : 0, g.accumulate);
 }
 
 // Fills the argument block shared by both tile sizes.
@@ -373,50 +489,79 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
     take = true;
   }
 
+  // ---- a last, partly filled round of tiles
+  // Unsplit tiles that do not fill a whole number of rounds leave a few CUs with one tile more than the
+  // rest, and those set the time: 576 tiles on 256 CUs take as long as 768 would.  When the tiles beyond
+  // the last whole round are at most half a round, they are cut into K ranges (of at least 8 K tiles) that
+  // spread over all CUs instead: 1536^3 forward 97 -> 77 us, 3072^3 587 -> 468 us.
+  long whole = 0;
+  Scratch partials(ctx);
+  if (splits == 1 && !ctx->fixed_mode) {
+    const long rounds = tiles / cus, rest = tiles - rounds * cus;
+    if (rounds >= 1 && rounds <= 8 && rest > 0 && 2 * rest <= cus) {
+      long s = cus / rest;
+      if (s > 16) s = 16;
+      if (s > total_ktiles / 8) s = total_ktiles / 8;
+      bool ok = s >= 2;
+      if (ok && wants_exchange(ctx, p)) {
+        ok = rest <= kTicketSlots &&
+             scratch_alloc(ctx, sizeof(float) * (size_t)rest * s * side * side, &partials.ptr) == PHIP_OK;
+        if (!ok) partials.ptr = nullptr;
+      }
+      if (ok) {
+        whole = rounds * cus;
+        splits = s;
+      }
+    }
+  }
+
   LdsArgs d;
   fill_args(p, side, splits, total_ktiles, a_bytes, b_bytes, ctx, &d);
-  Scratch partials(ctx);
-  if (splits > 1 && wants_exchange(ctx, p)) {
+  if (whole > 0) {
+    d.whole_tiles = (int)whole;
+    if (partials.ptr != nullptr) {
+      d.g.atomic = 2;
+      d.g.partial = static_cast<float *>(partials.ptr);
+      d.g.tickets = tile_tickets(ctx);
+    }
+  } else if (splits > 1 && wants_exchange(ctx, p)) {
     const int rc0 = prepare_split_exchange(ctx, p, tiles, (size_t)(256L << 20), &d.g, &partials);
     if (rc0 != PHIP_OK) return rc0;
   }
 
   int rc = PHIP_OK;
-  const unsigned grid = (unsigned)(tiles * splits);
-#define PHIP_LDS(SLOT, AK, BKM, SP)                                                                          \
+  const unsigned grid = (unsigned)(whole > 0 ? whole + (tiles - whole) * splits : tiles * splits);
+#define PHIP_LDS(SLOT, AK, BKM, MODE)                                                                        \
   do {                                                                                                       \
-    auto kern = gemm_f32_lds_kernel<AK, BKM, SP>;                                                            \
-    rc = raise_lds_limit(ctx, SLOT + (SP ? 3 : 0), reinterpret_cast<const void *>(kern), kLdsBytes);         \
+    auto kern = gemm_f32_lds_kernel<AK, BKM, MODE>;                                                          \
+    rc = raise_lds_limit(ctx, SLOT + (MODE == 2 ? kSlotGemmF32LdsMixed - kSlotGemmF32Lds : MODE == 1 ? 3 : 0), \
+                         reinterpret_cast<const void *>(kern), kLdsBytes);                                   \
     if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, ctx->stream, d);      \
   } while (0)
-#define PHIP_LDS64(AK, BKM, SP)                                                                              \
-  hipLaunchKernelGGL((gemm_f32_lds64_kernel<AK, BKM, SP>), dim3(grid), dim3(kThreads), kLds64Bytes, ctx->stream, d)
-  if (side == LBM) {
-    if (splits > 1) {
-      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, true);
-      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, true);
-      else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, true);
-    } else {
-      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, false);
-      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, false);
-      else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, false);
-    }
-  } else {
-    if (splits > 1) {
-      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64(false, true, true);
-      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64(false, false, true);
-      else PHIP_LDS64(true, true, true);
-    } else {
-      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64(false, true, false);
-      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64(false, false, false);
-      else PHIP_LDS64(true, true, false);
-    }
-  }
+#define PHIP_LDS64(AK, BKM, MODE)                                                                            \
+  hipLaunchKernelGGL((gemm_f32_lds64_kernel<AK, BKM, MODE>), dim3(grid), dim3(kThreads), kLds64Bytes, ctx->stream, d)
+#define PHIP_LDS_LAYOUTS(MODE)                                                                               \
+  do {                                                                                                       \
+    if (side == LBM) {                                                                                       \
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 0, false, true, MODE);                       \
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(kSlotGemmF32Lds + 1, false, false, MODE);                \
+      else PHIP_LDS(kSlotGemmF32Lds + 2, true, true, MODE);                                                  \
+    } else {                                                                                                 \
+      if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64(false, true, MODE);                                          \
+      else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64(false, false, MODE);                                   \
+      else PHIP_LDS64(true, true, MODE);                                                                     \
+    }                                                                                                        \
+  } while (0)
+  if (whole > 0) PHIP_LDS_LAYOUTS(2);
+  else if (splits > 1) PHIP_LDS_LAYOUTS(1);
+  else PHIP_LDS_LAYOUTS(0);
+#undef PHIP_LDS_LAYOUTS
 #undef PHIP_LDS
 #undef PHIP_LDS64
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
-  note_kernel(ctx, side == LBM ? (splits > 1 ? "f32_lds128_split" : "f32_lds128") : (splits > 1 ? "f32_lds64_split" : "f32_lds64"));
+  if (whole > 0) note_kernel(ctx, side == LBM ? "f32_lds128_mixed" : "f32_lds64_mixed");
+  else note_kernel(ctx, side == LBM ? (splits > 1 ? "f32_lds128_split" : "f32_lds128") : (splits > 1 ? "f32_lds64_split" : "f32_lds64"));
   *handled = true;
   return PHIP_OK;
 }

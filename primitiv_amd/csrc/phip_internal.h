@@ -245,6 +245,7 @@ enum LdsSlot {
   kSlotGemmF32StreamPair = 22,  // 1
   kSlotGemmH16Mid = 23,   // 6
   kSlotGemmH16Skinny = 29,  // 8
+  kSlotGemmF32LdsMixed = 37,  // 3
 };
 
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on

@@ -388,12 +388,44 @@ def test_midsize_long_k_f32(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(gb, rgb) <= F32_TOL
 
 
+# tiles that do not fill a whole number of rounds on the chip: the first rounds' tiles whole, the rest cut
+# into K ranges that spread over all compute units (partial tiles and tickets forward, atomics backward):
+# 64 x 64 tiles (576 = 2 x 256 + 64), ragged edges, a minibatch of products, and 128 x 128 tiles
+MIXED_F32 = [  # di, dj, dk, ba, bb
+    (1536, 1536, 1536, 1, 1),
+    (1540, 1000, 1530, 1, 1),
+    (520, 520, 640, 9, 9),
+    (2056, 2064, 2072, 1, 1),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", MIXED_F32)
+def test_partly_filled_last_round_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(di + 5 * dj + 7 * dk + ba)
+    bs = max(ba, bb)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+    ga0 = rng.standard_normal(a.size).astype(np.float32)
+    gb0 = rng.standard_normal(b.size).astype(np.float32)
+    dev.gemm_trace(True)
+    y, ga, gb = _fw_bw(dev, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    kernels = dev.gemm_trace(False)
+    assert any(k.endswith("_mixed") for k in kernels), kernels   # (listed per stream, not in call order)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    assert norm_rel_err(y, ry) <= F32_TOL
+    assert norm_rel_err(ga, rga) <= F32_TOL
+    assert norm_rel_err(gb, rgb) <= F32_TOL
+
+
 # an overwriting product with few output tiles and a long K is cut between workgroups
 # that meet through partial tiles, summed in a fixed order by whichever finishes last:
 # right, and the same bits on every run
 @pytest.mark.parametrize("di,dj,dk,ba,bb", [(256, 784, 1, 1, 128), (64, 3000, 1, 1, 40), (100, 5000, 33, 1, 1),
                                             (48, 2048, 8, 3, 3), (1028, 2052, 1100, 1, 1),
-                                            (1024, 4096, 1, 1, 128)])
+                                            (1024, 4096, 1, 1, 128), (1536, 1536, 1536, 1, 1),
+                                            (520, 520, 640, 9, 9)])
 def test_split_forward_is_right_and_reproducible(dev, di, dj, dk, ba, bb):
     rng = np.random.default_rng(di + dj)
     a = rng.standard_normal(di * dj * ba).astype(np.float32)
@@ -441,7 +473,7 @@ def test_few_outputs_long_k_forward_f32(dev, di, dj, dk, ba, bb):
 # ragged shapes, per-sample products and a contraction over the minibatch
 SPLIT_BW = [(256, 784, 1, 1, 128), (2048, 512, 1, 1, 64), (4100, 650, 1, 1, 64), (10000, 650, 1, 1, 64),
             (1028, 2052, 1100, 1, 1), (1536, 512, 4096, 1, 1), (96, 1000, 5, 1, 3), (48, 2048, 8, 3, 3),
-            (300, 20, 5, 9, 1), (130, 70, 258, 1, 4)]
+            (300, 20, 5, 9, 1), (130, 70, 258, 1, 4), (1536, 1536, 1536, 1, 1), (1540, 1000, 1530, 1, 1)]
 
 
 @pytest.mark.parametrize("di,dj,dk,ba,bb", SPLIT_BW)
