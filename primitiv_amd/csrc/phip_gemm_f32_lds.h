@@ -62,10 +62,11 @@ __device__ inline void lds_dma_b32(uint4v rsrc, uint32_t lds_addr, uint32_t voff
 }
 
 // The wave's load instructions (1 KiB of LDS each) for one operand tile of
-// ROWS rows or columns by 32 k: ROWS / 32 per wavefront.
-template <bool KMAJOR, int ROWS = 128>
+// ROWS rows or columns by 32 k: ROWS / 32 per wavefront of a workgroup of four
+// (ROWS / 8 between the WAVES wavefronts of the workgroup).
+template <bool KMAJOR, int ROWS = 128, int WAVES = 4>
 struct DmaLoader {
-  static constexpr int kInstr = ROWS / 32;
+  static constexpr int kInstr = ROWS / 8 / WAVES;
   static constexpr int kLanesPerRow = ROWS / 4;  // (m/n-contiguous) lanes that cover one k row
   uint32_t off[kInstr];  // byte offset of this lane's chunk per instruction, at K tile 0
   uint32_t step;         // bytes per K tile

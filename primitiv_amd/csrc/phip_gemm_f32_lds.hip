@@ -408,6 +408,130 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsAr
   emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, tw.shared ? g.atomic : 0, g.accumulate);
 }
 
+// 64 x 64 tiles without a barrier in the K loop, for a launch that gives every CU at most one workgroup.
+// With one workgroup on a CU nothing overlaps the wait at a barrier (timestamps in a variant of the kernel
+// above with eight wavefronts: of the 1850 cycles that a K tile takes, 480 are the wait for loads plus the
+// barrier, and the matrix pipe of a SIMD is busy 1024), so here no wavefront shares LDS with another: each
+// of the eight wavefronts of a workgroup (two per SIMD) moves its own
+// operands - the 32 rows of A and the 32 columns of B of its block, 32 k at a time, 8 KiB per stage, two
+// stages - into its own 16 KiB of LDS and waits only for its own loads.  Wavefronts w and w + 4 share a
+// block and take alternate K tiles; their tiles meet through LDS at the end.  Each wavefront alternates
+// between two accumulators, so that a matrix instruction never waits for the result of the one before it.  An operand block is loaded by
+// the two wavefront pairs that need it, twice the bytes from L2 (32 B / clk / CU), which the loads that
+// write LDS directly deliver.
+constexpr int kThreads64w = 512;
+constexpr int kLds64wBytes = 8 * 16384;
+
+template <bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(kThreads64w, 2) void gemm_f32_lds64w_kernel(const LdsArgs d) {
+  const GemmArgs &g = d.g;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kh = wave >> 2;  // K tiles kh, kh + 2, ...
+  const int wm = wave & 1, wn = (wave >> 1) & 1;
+
+  const TileWork tw = tile_work<0>(d);
+  const int tile_m = tw.tile_m, tile_n = tw.tile_n, z = tw.z;
+  const int m0 = tile_m * SBM, n0 = tile_n * SBN;
+  const int row0 = m0 + wm * 32, col0 = n0 + wn * 32;
+
+  DmaLoader<A_KMAJOR, 32, 1> la;
+  DmaLoader<B_KMAJOR, 32, 1> lb;
+  la.init(g.lda, row0, g.M, 0, lane);
+  lb.init(g.ldb, col0, g.N, 0, lane);
+  FragReaderF<A_KMAJOR, 32> fra;
+  FragReaderF<B_KMAJOR, 32> frb;
+  fra.init(0, lane);
+  frb.init(0, lane);
+
+  const float *Az = g.A + (long)z * g.sA;
+  const float *Bz = g.B + (long)z * g.sB;
+
+  float16v acc0, acc1;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.0f;
+
+  constexpr int kOwnRegion = 4096, kOwnStage = 2 * kOwnRegion;
+  unsigned char *own = lds + wave * (2 * kOwnStage);
+  const uint32_t own_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)own;
+  const int own_tiles = (g.total_ktiles - kh + 1) / 2;
+  auto issue_tile = [&](int t, int into, int q) {
+    // instruction q of the 8 (4 for A, then 4 for B) that move this wavefront's K tile t into stage `into`
+    const bool live = t < own_tiles;
+    const int ktc = live ? 2 * t + kh : 0;
+    const int r = ktc / g.ktiles_per_r;
+    const int kt_in_r = ktc - r * g.ktiles_per_r;
+    const uint32_t stage = own_base + (uint32_t)into * kOwnStage;
+    if (q < 4) la.issue(make_rsrc_words(Az + (long)r * g.rA, d.a_bytes), stage, 0, q, kt_in_r, g.K, live);
+    else lb.issue(make_rsrc_words(Bz + (long)r * g.rB, d.b_bytes), stage + kOwnRegion, 0, q - 4, kt_in_r, g.K, live);
+  };
+
+#pragma unroll
+  for (int q = 0; q < 8; ++q) issue_tile(0, 0, q);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) issue_tile(1, 1, q);
+  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // tile 0 has landed
+
+  float fa[2][2][4], fb[2][2][4];
+  constexpr int kReadsA = A_KMAJOR ? 1 : 4, kReadsB = B_KMAJOR ? 1 : 4;
+#pragma unroll
+  for (int q = 0; q < kReadsA; ++q) fra.read_one(own, 0, q, fa[0]);
+#pragma unroll
+  for (int q = 0; q < kReadsB; ++q) frb.read_one(own + kOwnRegion, 0, q, fb[0]);
+
+  for (int t = 0; t < own_tiles; ++t) {
+    const int stage = t & 1;
+#pragma unroll
+    for (int gk = 0; gk < 4; ++gk) {
+      const int cur = gk & 1, nxt = cur ^ 1;
+      const unsigned char *src = own + (gk < 3 ? stage : stage ^ 1) * kOwnStage;
+      const int ngk = gk < 3 ? gk + 1 : 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // rows of the instruction's result follow n, its columns follow m
+        if (e & 1) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][0][e], fa[cur][0][e], acc1, 0, 0, 0);
+        else acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][0][e], fa[cur][0][e], acc0, 0, 0, 0);
+        if (e < kReadsA) fra.read_one(src, ngk, e, fa[nxt]);
+        if (e < kReadsB) frb.read_one(src + kOwnRegion, ngk, e, fb[nxt]);
+        // tile t + 2 refills this stage: every read of it was waited for behind group 2
+        if (gk == 3) {
+          issue_tile(t + 2, stage, 2 * e);
+          issue_tile(t + 2, stage, 2 * e + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // the loads of tile t + 1 have landed and the reads of this stage are done
+      if (gk == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+  // the upper four wavefronts hand their tiles to the lower four through their own LDS
+  float16v acc = acc0 + acc1;
+  if (kh == 1) {
+    float *red = reinterpret_cast<float *>(own);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[v * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+  if (kh == 1) return;
+
+  const float *red = reinterpret_cast<const float *>(lds + (wave + 4) * (2 * kOwnStage));
+  float *Cz = g.C + (long)z * g.sC;
+  const bool interior = m0 + SBM <= g.M && n0 + SBN <= g.N;
+  int ns[16];
+  float vals[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    ns[v] = 8 * (v / 4) + (v % 4);
+    vals[v] = acc[v] + red[v * 64 + lane];
+  }
+  emit_c<16>(Cz, g.ldc, row0, col0, lane, g.M, g.N, interior, ns, vals, 0, g.accumulate);
+}
+
 // Fills the argument block shared by both tile sizes.
 static void fill_args(const Gemm &p, int side, long splits, long total_ktiles, long a_bytes, long b_bytes,
                       phip_ctx *ctx, LdsArgs *d) {
@@ -493,7 +617,7 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
   // Unsplit tiles that do not fill a whole number of rounds leave a few CUs with one tile more than the
   // rest, and those set the time: 576 tiles on 256 CUs take as long as 768 would.  When the tiles beyond
   // the last whole round are at most half a round, they are cut into K ranges (of at least 8 K tiles) that
-  // spread over all CUs instead: 1536^3 forward 97 -> 77 us, 3072^3 587 -> 468 us.
+  // spread over all CUs instead: 3072^3 forward 587 -> 478 us, both gradients 1146 -> 856 us.
   long whole = 0;
   Scratch partials(ctx);
   if (splits == 1 && !ctx->fixed_mode) {
@@ -552,7 +676,20 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
       else PHIP_LDS64(true, true, MODE);                                                                     \
     }                                                                                                        \
   } while (0)
-  if (whole > 0) PHIP_LDS_LAYOUTS(2);
+  // one workgroup per CU at most: the kernel whose wavefronts do not wait for each other
+  const bool alone = side == SBM && splits == 1 && whole == 0 && tiles <= cus;
+  if (alone) {
+#define PHIP_LDS64W(SLOT, AK, BKM)                                                                           \
+  do {                                                                                                       \
+    auto kern = gemm_f32_lds64w_kernel<AK, BKM>;                                                             \
+    rc = raise_lds_limit(ctx, kSlotGemmF32Lds64w + (SLOT), reinterpret_cast<const void *>(kern), kLds64wBytes); \
+    if (rc == PHIP_OK) hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads64w), kLds64wBytes, ctx->stream, d); \
+  } while (0)
+    if (!p.a_kmajor && p.b_kmajor) PHIP_LDS64W(0, false, true);
+    else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS64W(1, false, false);
+    else PHIP_LDS64W(2, true, true);
+#undef PHIP_LDS64W
+  } else if (whole > 0) PHIP_LDS_LAYOUTS(2);
   else if (splits > 1) PHIP_LDS_LAYOUTS(1);
   else PHIP_LDS_LAYOUTS(0);
 #undef PHIP_LDS_LAYOUTS
@@ -560,7 +697,8 @@ int gemm_f32_lds(phip_ctx *ctx, const Gemm &p, bool *handled) {
 #undef PHIP_LDS64
   if (rc != PHIP_OK) return rc;
   PHIP_LAUNCH_CHECK();
-  if (whole > 0) note_kernel(ctx, side == LBM ? "f32_lds128_mixed" : "f32_lds64_mixed");
+  if (alone) note_kernel(ctx, "f32_lds64w");
+  else if (whole > 0) note_kernel(ctx, side == LBM ? "f32_lds128_mixed" : "f32_lds64_mixed");
   else note_kernel(ctx, side == LBM ? (splits > 1 ? "f32_lds128_split" : "f32_lds128") : (splits > 1 ? "f32_lds64_split" : "f32_lds64"));
   *handled = true;
   return PHIP_OK;

@@ -246,6 +246,7 @@ enum LdsSlot {
   kSlotGemmH16Mid = 23,   // 6
   kSlotGemmH16Skinny = 29,  // 8
   kSlotGemmF32LdsMixed = 37,  // 3
+  kSlotGemmF32Lds64w = 40,    // 3
 };
 
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on

@@ -388,6 +388,35 @@ def test_midsize_long_k_f32(dev, di, dj, dk, ba, bb):
     assert norm_rel_err(gb, rgb) <= F32_TOL
 
 
+# an overwriting product with at most one 64 x 64 tile per compute unit: eight wavefronts per tile, each with
+# its own operand blocks in LDS and no barrier in the K loop, pairs of wavefronts taking alternate K tiles -
+# a K of five K tiles, an odd number of them, not a multiple of 32; ragged M and N; a minibatch on the grid
+# and one folded into the columns
+ALONE_F32 = [  # di, dj, dk, ba, bb
+    (1024, 1024, 1024, 1, 1),
+    (768, 800, 776, 1, 1),
+    (1000, 132, 520, 1, 1),
+    (1000, 160, 1020, 1, 1),
+    (520, 1036, 264, 3, 3),
+    (776, 2000, 200, 1, 4),
+]
+
+
+@pytest.mark.parametrize("di,dj,dk,ba,bb", ALONE_F32)
+def test_one_tile_per_compute_unit_f32(dev, di, dj, dk, ba, bb):
+    rng = np.random.default_rng(3 * di + dj + 11 * dk + ba)
+    a = rng.standard_normal(di * dj * ba).astype(np.float32)
+    b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+    ta = dev.new_tensor_by_vector(pa.Shape([di, dj], ba), a)
+    tb = dev.new_tensor_by_vector(pa.Shape([dj, dk], bb), b)
+    dev.gemm_trace(True)
+    y = dev.matmul_fw(ta, tb).to_vector()
+    assert dev.gemm_trace(False) == ["f32_lds64w"]
+    assert norm_rel_err(y, oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)) <= F32_TOL
+    for _ in range(5):
+        assert np.array_equal(dev.matmul_fw(ta, tb).to_vector(), y)
+
+
 # tiles that do not fill a whole number of rounds on the chip: the first rounds' tiles whole, the rest cut
 # into K ranges that spread over all compute units (partial tiles and tickets forward, atomics backward):
 # 64 x 64 tiles (576 = 2 x 256 + 64), ragged edges, a minibatch of products, and 128 x 128 tiles
