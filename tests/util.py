@@ -18,6 +18,17 @@ def ulp_diff(a, b):
     return np.abs(ia - ib)
 
 
+def round_to_storage(x, storage):
+    """float32 values rounded once, to nearest even, to the 16-bit storage type ("f16" / "bf16"), as float32."""
+    x = np.asarray(x, dtype=np.float32)
+    if storage == "f16":
+        with np.errstate(over="ignore"):
+            return x.astype(np.float16).astype(np.float32)
+    bits = x.view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32)
+
+
 def vector_match(expected, actual, ulps=4):
     expected = np.asarray(expected, dtype=np.float32).reshape(-1)
     actual = np.asarray(actual, dtype=np.float32).reshape(-1)
