@@ -411,6 +411,8 @@ constexpr int SM = 32, SN = 32;
 constexpr int kRegionS = 32 * BK * 2;  // bytes of one operand's K tile: 32 rows (m or n) x 64 k
 constexpr int kStageS = 2 * kRegionS;
 constexpr int kMaxStagesS = 18;        // 144 KiB
+constexpr int kRoundS = 9;             // a longer K range is walked in rounds of this many K tiles, two rounds resident
+constexpr int kMaxRoundsS = 5;
 constexpr int kReduceBytesS = 16384;   // the four wavefronts' tiles, when they are added up
 
 // One piece (16 bytes per lane) of each of eight partial tiles, all in flight at once, and the wait.
@@ -505,12 +507,25 @@ __device__ inline void skinny_tile_small(const SkinnyArgs &g, unsigned char *lds
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
   const uint16_t *Az = g.A + (long)z * g.sA;
   const uint16_t *Bz = g.B + (long)z * g.sB;
-  {
-    int r = kb / g.ktiles_per_r, kin = kb - r * g.ktiles_per_r;
-    for (int s = 0; s < n_st; ++s) {
+  // after the sum over the wavefronts, wavefront w owns the 16 x 16 block (w / 2, w % 2) of the tile
+  uint16_t *Cz = g.C + (long)z * g.sC;
+  const int g4 = lane >> 4, nl = lane & 15;
+  const int m = m0 + 16 * (wave >> 1) + 4 * g4;
+  const int n = n0 + 16 * (wave & 1) + nl;
+  // C's old values first: they have the longest way to come, and as the oldest load they are covered by
+  // every wait for operands below
+  uint2v old = {0u, 0u};
+  if (g.accumulate && g.vec_c && n < g.N && m + 4 <= g.M) old = *reinterpret_cast<const uint2v *>(Cz + m + (long)n * g.ldc);
+
+  // K tiles [first, first + count) of the workgroup's range into LDS from `slot` on: two loads per wavefront
+  // and K tile
+  auto issue_stages = [&](int first, int count, int slot) {
+    const int kt = kb + first;
+    int r = kt / g.ktiles_per_r, kin = kt - r * g.ktiles_per_r;
+    for (int s = 0; s < count; ++s) {
       const uint4v ra = make_rsrc_words(Az + (long)r * g.rA, g.a_bytes);
       const uint4v rb = make_rsrc_words(Bz + (long)r * g.rB, g.b_bytes);
-      const uint32_t stage = lds_base + (uint32_t)s * kStageS;
+      const uint32_t stage = lds_base + (uint32_t)(slot + s) * kStageS;
       la.issue(ra, stage, wave, kin, g.K);
       lb.issue(rb, stage + kRegionS, wave, kin, g.K);
       if (++kin == g.ktiles_per_r) {
@@ -518,30 +533,38 @@ __device__ inline void skinny_tile_small(const SkinnyArgs &g, unsigned char *lds
         ++r;
       }
     }
-  }
-  // after the sum over the wavefronts, wavefront w owns the 16 x 16 block (w / 2, w % 2) of the tile
-  uint16_t *Cz = g.C + (long)z * g.sC;
-  const int g4 = lane >> 4, nl = lane & 15;
-  const int m = m0 + 16 * (wave >> 1) + 4 * g4;
-  const int n = n0 + 16 * (wave & 1) + nl;
-  uint2v old = {0u, 0u};
-  if (g.accumulate && g.vec_c && n < g.N && m + 4 <= g.M) old = *reinterpret_cast<const uint2v *>(Cz + m + (long)n * g.ldc);
+  };
+  // A range of at most kMaxStagesS K tiles is resident at once: one round of loads, one wait.  A longer one
+  // is walked in rounds of kRoundS K tiles through two halves of LDS, the loads of round r + 1 in flight
+  // under the matrix instructions of round r.
+  const bool one_round = n_st <= kMaxStagesS;
+  const int per_round = one_round ? n_st : kRoundS;
+  const int rounds = one_round ? 1 : (n_st + kRoundS - 1) / kRoundS;
+  issue_stages(0, per_round, 0);
+  if (rounds > 1) issue_stages(kRoundS, n_st - kRoundS < kRoundS ? n_st - kRoundS : kRoundS, kRoundS);
+
   float4v acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
 
-  {
+  const bool ragged = (A_KMAJOR || B_KMAJOR) && (g.K & 7) != 0;
+  const int kin0 = kb % g.ktiles_per_r;
+  for (int rd = 0; rd < rounds; ++rd) {
+    const int done = rd * per_round;                       // K tiles of the rounds before
+    const int count = n_st - done < per_round ? n_st - done : per_round;
+    // loads return in order: with a whole round (2 kRoundS loads per wavefront) behind it, round rd has landed
+    // when that many are still on their way
+    if (rd + 1 < rounds && n_st - done - per_round >= kRoundS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kRoundS) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const uint32_t half = lds_base + (uint32_t)((rd & 1) * kRoundS) * kStageS;
     // k steps of 32: wavefront w takes steps w, w + 4, ... of the workgroup's range
-    const bool ragged = (A_KMAJOR || B_KMAJOR) && (g.K & 7) != 0;
-    const int kin0 = kb % g.ktiles_per_r;
-    for (int ks = wave; ks < 2 * n_st; ks += 4) {
+    for (int ks = (wave - 2 * done) & 3; ks < 2 * count; ks += 4) {
       const int s = ks >> 1, tt = ks & 1;
-      const uint32_t stage = lds_base + (uint32_t)s * kStageS;
-      const int kin = (kin0 + s) % g.ktiles_per_r;
+      const uint32_t stage = half + (uint32_t)s * kStageS;
+      const int kin = (kin0 + done + s) % g.ktiles_per_r;
       uint4v fa[2], fb[2];
 #pragma unroll
       for (int i = 0; i < 2; ++i) fa[i] = read_fragment_small<A_KMAJOR>(stage, 16 * i, tt, lane);
@@ -563,6 +586,12 @@ __device__ inline void skinny_tile_small(const SkinnyArgs &g, unsigned char *lds
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma<BF16>(fa[i], fb[j], acc[i][j]);
+    }
+    if (rd + 2 < rounds) {
+      // round rd + 2 takes this round's half once every wavefront has read what it needed from it
+      __syncthreads();
+      const int next = (rd + 2) * kRoundS;
+      issue_stages(next, n_st - next < kRoundS ? n_st - next : kRoundS, (rd & 1) * kRoundS);
     }
   }
   // the four wavefronts' tiles, added in the order of the wavefronts: wavefront w sums block w
@@ -689,21 +718,26 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
 
   // Tile shape and stages per workgroup: the choice that a small cost model likes best (microseconds): the
   // loads of the workgroups that share a compute unit (about 0.4 per 16 KiB), the exchange of partial tiles
-  // when K is cut (store, ticket, then one round trip through memory per four - small tiles: eight - ranges),
-  // the sum over the wavefronts of a small tile, and a second round of workgroups if the grid does not fit
-  // the chip at once.  Ties go to the large tiles, which load each operand fewer times.
+  // when K is cut (store, ticket: 2; then 2 per round trip through memory, one per four - small tiles: eight -
+  // ranges: `gx = W^T gy` of the output projection, 20 ranges in five round trips, measured 16.4 us), the sum
+  // over the wavefronts of a small tile, 1 for every further round of a range that LDS does not hold at once,
+  // and a second round of workgroups if the grid does not fit the chip at once.  Ties go to the large tiles,
+  // which load each operand fewer times.
   int best_s = 0, best_small = 0;
   long best_tiles = 0;
   double best = 0.0;
   for (int small = 0; small < 2; ++small) {
-    const int side = small ? SM : TM, stage_bytes = small ? kStageS : kStage, max_s = small ? kMaxStagesS : kMaxStages;
+    // (a small tile's range may exceed what LDS holds: it is then walked in rounds of kRoundS K tiles)
+    const int side = small ? SM : TM, stage_bytes = small ? kStageS : kStage;
+    const int max_s = small ? kRoundS * kMaxRoundsS : kMaxStages;
     const long tiles = (long)((p.M + side - 1) / side) * ((p.N + side - 1) / side) * p.batch;
     if (tiles > kTicketSlots) continue;
     for (int s = 1; s <= max_s; ++s) {
       const long splits = (total_ktiles + s - 1) / s;
       const int s_eff = (int)((total_ktiles + splits - 1) / splits);
       if (s_eff != s && s != max_s) continue;  // the same cut as a smaller s
-      int lds = s_eff * stage_bytes;
+      const int rounds_of = small && s_eff > kMaxStagesS ? (s_eff + kRoundS - 1) / kRoundS : 1;
+      int lds = (rounds_of > 1 ? kMaxStagesS : s_eff) * stage_bytes;
       if (small && lds < kReduceBytesS) lds = kReduceBytesS;
       int occ = (160 * 1024) / lds;
       if (occ > 4) occ = 4;  // registers: four wavefronts per SIMD
@@ -717,8 +751,8 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
       long per_cu = (grid + cus - 1) / cus;
       if (per_cu > occ) per_cu = occ;
       const double loads = 0.4 * s_eff * per_cu * stage_bytes / kStage;
-      const double exchange = splits > 1 ? 2.0 + 1.2 * ((splits + (small ? 7 : 3)) / (small ? 8 : 4)) : 0.0;
-      const double cost = rounds * (1.0 + (small ? 0.3 : 0.0) + loads) + exchange;
+      const double exchange = splits > 1 ? 2.0 + 2.0 * ((splits + (small ? 7 : 3)) / (small ? 8 : 4)) : 0.0;
+      const double cost = rounds * (1.0 + (small ? 0.3 : 0.0) + loads + 1.0 * (rounds_of - 1)) + exchange;
       if (best_s == 0 || cost < best - 1e-9) {
         best = cost;
         best_s = s_eff;
@@ -755,7 +789,7 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
   plan->tiles = tiles;
   plan->grid = tiles * splits;
   plan->stages = (int)((total_ktiles + splits - 1) / splits);
-  plan->lds = plan->stages * (best_small ? kStageS : kStage);
+  plan->lds = (best_small && plan->stages > kMaxStagesS ? kMaxStagesS : plan->stages) * (best_small ? kStageS : kStage);
   if (best_small && plan->lds < kReduceBytesS) plan->lds = kReduceBytesS;
   plan->tile_floats = side * side;
   return true;
