@@ -37,13 +37,13 @@ STORAGE_CODE = {"f32": 0, "f16": 1, "bf16": 2}
 # y += x of known size in the same runs), summed over a step's launches ("HBM bytes per step by the
 # counters" there).  Algorithmic bytes for comparison are Workload.bytes_per_step().
 COUNTER_TRAFFIC_BYTES_PER_STEP = {
-    "square_batched": 762.6e6,       # 206.23 + 284.09 + 272.26 MB: the three gemm_f32_lds_kernel launches
+    "square_batched": 762.9e6,       # the three gemm_f32_lds_kernel launches: 206 + 284 + 272 MB: the three gemm_f32_lds_kernel launches
     "dense": 14.58e6,                # gemm_f32_tile16_kernel 7.06 + gemm_f32_pair_kernel 7.52 MB
-    "rnn_gate": 873.0e6,             # 30 x (9.64 + 19.47 MB)
-    "output_projection": 4468.9e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.03 MB)
-    "half_storage": 6284.7e6,        # 2 x 2122.68 + 1972.15 + 67.17 MB (transposed copy of a)
-    "rnn_gate:f16": 486.9e6,         # 30 x (gemm_h16_skinny_kernel 4.83 + gemm_h16_skinny_pair_kernel 11.40 MB)
-    "output_projection:f16": 3150.3e6,  # 35 x (30.44 + 36.69 + 22.88 MB: three gemm_h16_skinny_kernel launches)
+    "rnn_gate": 872.4e6,             # 30 x (9.64 + 19.44 MB)
+    "output_projection": 4469.8e6,   # 35 x (gemm_f32_slab_kernel 34.65 + gemm_f32_stream_pair_kernel 93.06 MB)
+    "half_storage": 6293.6e6,        # two launches of 2.12 GB, one of 1.98 GB, 67 MB for the transposed copy of a
+    "rnn_gate:f16": 487.4e6,         # 30 x (gemm_h16_skinny_kernel 4.83 + gemm_h16_skinny_pair_kernel 11.41 MB)
+    "output_projection:f16": 3284.8e6,  # 35 x (30.46 + 36.68 + 26.71 MB: three gemm_h16_skinny_kernel launches)
 }
 # per launch of the headline kernel (average of its three operand-layout instantiations)
 HEADLINE_TRAFFIC_BYTES = COUNTER_TRAFFIC_BYTES_PER_STEP["square_batched"] / 3
