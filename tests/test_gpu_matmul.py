@@ -671,6 +671,44 @@ def test_per_timestep_shapes_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
     assert np.array_equal(y2, y) and np.array_equal(ga2, ga) and np.array_equal(gb2, gb)     # and the same bits
 
 
+# a long contraction against few output tiles: K ranges of more than 18 K tiles, which the 32 x 32 tiles walk in
+# rounds through two halves of LDS - K not a multiple of 64 or of 8, a contraction that runs over the
+# minibatch (its K tiles restart with every sample), one to five rounds, with and without a cut between workgroups
+LONG_K_H16 = [  # di, dj, dk, ba, bb
+    (34, 5000, 20, 1, 1),
+    (40, 2890, 30, 1, 1),
+    (650, 10000, 1, 1, 20),
+    (96, 1234, 64, 1, 1),
+    (20, 1300, 2, 1, 64),
+    (1300, 130, 48, 9, 1),
+    (3000, 64, 64, 1, 1),
+    (2600, 34, 36, 3, 1),
+]
+
+
+@pytest.mark.parametrize("which", ["f16", "bf16"])
+@pytest.mark.parametrize("di,dj,dk,ba,bb", LONG_K_H16)
+def test_long_k_narrow_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
+    d = dev16 if which == "f16" else devbf16
+    rng = np.random.default_rng(7 * di + dj + 13 * dk + ba)
+    bs = max(ba, bb)
+    r16 = (lambda x: x.astype(np.float16).astype(np.float32)) if which == "f16" else \
+        (lambda x: (x.view(np.uint32) & 0xFFFF0000).view(np.float32))
+    a = r16(rng.standard_normal(di * dj * ba).astype(np.float32))
+    b = r16(rng.standard_normal(dj * dk * bb).astype(np.float32))
+    gy = r16(rng.standard_normal(di * dk * bs).astype(np.float32))
+    ga0 = r16(rng.standard_normal(a.size).astype(np.float32))
+    gb0 = r16(rng.standard_normal(b.size).astype(np.float32))
+    y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    ry = oracle.matmul_fw(a, b, di, dj, dk, ba, bb, 8)
+    rga, rgb = oracle.matmul_bw(a, b, gy, ga0, gb0, di, dj, dk, ba, bb, 8)
+    ulp = 2.0 ** -10 if which == "f16" else 2.0 ** -7
+    for name, got, ref in (("y", y, ry), ("ga", ga, rga), ("gb", gb, rgb)):
+        assert norm_rel_err(got, ref) <= ulp, name
+    y2, ga2, gb2 = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+    assert np.array_equal(y2, y) and np.array_equal(ga2, ga) and np.array_equal(gb2, gb)
+
+
 def test_f16_matches_oracle_on_rounded_inputs(dev16):
     # With inputs already representable in fp16 the only error left is the
     # final rounding of the output (<= 2^-11 relative per element) on top of
