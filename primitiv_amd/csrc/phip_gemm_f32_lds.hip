@@ -6,10 +6,12 @@
 // v_mfma_f32_32x32x2_f32 tiles.  Two 32 KiB LDS stages (A region then B region,
 // 16 KiB each); two workgroups share a CU.
 //
-// SPLIT: a problem with too few output tiles for the chip cuts its K range
+// MODE 1: a problem with too few output tiles for the chip cuts its K range
 // between workgroups; an accumulating product adds its tiles into C with fp32
 // atomics, an overwriting one meets through partial tiles and a per-tile
-// ticket (see last_of_tile).  The unsplit instantiation carries none of that.
+// ticket (see last_of_tile).  MODE 2: only the tiles of a partly filled last
+// round are cut (see TileWork).  The unsplit instantiation (MODE 0) carries
+// none of that.
 //
 // The LDS image of an operand tile is described with the loader that builds it.
 #include "phip_gemm_f32_lds.h"
@@ -114,7 +116,6 @@ __device__ inline void sum_tile_partials(const float *P, int splits, int row0, i
 // MODE 0: unsplit, 1: every tile shared by K ranges, 2: mixed (see TileWork).
 template <bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void gemm_f32_lds_kernel(const LdsArgs d) {
-  constexpr bool SPLIT = MODE != 0;
   const GemmArgs &g = d.g;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
@@ -288,7 +289,6 @@ constexpr int kLds64Bytes = 2 * kStage64;
 
 template <bool A_KMAJOR, bool B_KMAJOR, int MODE>
 __global__ __launch_bounds__(kThreads, 4) void gemm_f32_lds64_kernel(const LdsArgs d) {
-  constexpr bool SPLIT = MODE != 0;
   const GemmArgs &g = d.g;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
