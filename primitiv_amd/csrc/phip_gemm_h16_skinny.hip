@@ -702,7 +702,11 @@ bool plan_skinny(const phip_ctx *ctx, const Gemm &p, SkinnyPlan *plan, int place
   if (p.a_kmajor && !p.b_kmajor) return false;
   if (p.M < 1 || p.N < 1 || p.K < 16) return false;
   // the narrow side: at most 128 columns or rows of output, or a short K (a rank-K update)
-  const bool narrow = p.N <= 128 || p.M <= 128 || p.K <= 128;
+  // ... or an output of at most half a million elements: such a product is a launch of a few microseconds whatever its K, and one
+  // round of loads beats the staged loop (512^3: forward 6.8 -> 4.5 us, both gradients in one launch 13.7 -> 5.6;
+  // 800 x 784 by 200 columns 9.8 -> 5.4 and 18.2 -> 10.1); from 768^3 on the 128 x 128 tiles are ahead (8.8
+  // against 9.7 us)
+  const bool narrow = p.N <= 128 || p.M <= 128 || p.K <= 128 || (long)p.M * p.N * p.batch <= 512L * 1024L;
   if (!narrow) return false;
   // 16-byte loads from 4-byte aligned addresses: even leading dimensions and strides, aligned bases
   if (reinterpret_cast<uintptr_t>(p.A) % 16 != 0 || reinterpret_cast<uintptr_t>(p.B) % 16 != 0) return false;
