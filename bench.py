@@ -386,21 +386,36 @@ def measure_pointwise(reps=20):
     operation needs read once, every result written once, a gradient read and written)
     over the event time, against the 8 TB/s HBM peak.  Large cases are 64 Mi elements per
     tensor; the bias cases use a 1 Mi-element bias over a minibatch of 64, and the
-    recurrent-layer shape (2048 x 64) shows the latency floor."""
+    recurrent-layer shape (2048 x 64) shows the latency floor.
+    The large cases walk round several sets of operands, so that no call finds its operands in the 256 MB
+    Infinity Cache from the call before: repeated over ONE set, a copy of 256 MiB reads 5.4 TB/s, the same copy
+    with streaming stores 8.6 TB/s (the source then stays in the cache between calls), and one of 1 GiB 5.1
+    either way - the rate of HBM is what the rotation shows."""
     S = pa.Shape
     out = []
+    SETS = 4
+
+    class Ring:
+        """SETS tensors of one shape, handed out in turn."""
+        def __init__(self, make):
+            self.t, self.i = [make() for _ in range(SETS)], 0
+
+        def __call__(self):
+            self.i = (self.i + 1) % SETS
+            return self.t[self.i]
+
     for storage, item in (("f32", 4), ("f16", 2)):
         dev = pa.HIP(0) if storage == "f32" else pa.HIP16(0, storage=storage)
         n = 64 << 20
-        x = dev.new_tensor_by_constant(S([n]), 0.5)
-        y = dev.new_tensor_by_constant(S([n]), 0.25)
-        g = dev.new_tensor_by_constant(S([n]), 0.0)
-        g2 = dev.new_tensor_by_constant(S([n]), 0.0)
+        xs = Ring(lambda: dev.new_tensor_by_constant(S([n]), 0.5))
+        ys = Ring(lambda: dev.new_tensor_by_constant(S([n]), 0.25))
+        gs = Ring(lambda: dev.new_tensor_by_constant(S([n]), 0.0))
+        g2s = Ring(lambda: dev.new_tensor_by_constant(S([n]), 0.0))
         vol, bs = 1 << 20, 64
         bias = dev.new_tensor_by_constant(S([vol]), 0.5)
         gbias = dev.new_tensor_by_constant(S([vol]), 0.0)
-        xb = dev.new_tensor_by_constant(S([vol], bs), 0.5)
-        gxb = dev.new_tensor_by_constant(S([vol], bs), 0.0)
+        xbs = Ring(lambda: dev.new_tensor_by_constant(S([vol], bs), 0.5))
+        gxbs = Ring(lambda: dev.new_tensor_by_constant(S([vol], bs), 0.0))
         sv, sb = 2048, 64
         sbias = dev.new_tensor_by_constant(S([sv]), 0.5)
         sx = dev.new_tensor_by_constant(S([sv], sb), 0.5)
@@ -408,15 +423,16 @@ def measure_pointwise(reps=20):
         sgb = dev.new_tensor_by_constant(S([sv]), 0.0)
         big, med = n * item, vol * bs * item
         cases = [
-            ("tanh_fw", lambda: dev.unary_fw("tanh", x), 2 * big),
-            ("tanh_bw", lambda: dev.unary_bw("tanh", x, y, x, g), 4 * big),
-            ("prelu_fw", lambda: dev.const_fw("prelu", x, 0.01), 2 * big),
-            ("add_fw", lambda: dev.binary_fw("add", x, y), 3 * big),
-            ("multiply_bw", lambda: dev.binary_bw("multiply", x, y, x, y, g, g2), 7 * big),
-            ("bias_add_fw", lambda: dev.binary_fw("add", xb, bias), 2 * med + vol * item),
-            ("bias_add_bw", lambda: dev.binary_bw("add", xb, bias, xb, xb, gxb, gbias), 3 * med + 2 * vol * item),
-            ("inplace_add", lambda: dev.inplace_add(x, y), 3 * big),
-            ("inplace_multiply_const", lambda: dev.inplace_multiply_const(1.0, y), 2 * big),
+            ("tanh_fw", lambda: dev.unary_fw("tanh", xs()), 2 * big),
+            ("tanh_bw", lambda: (lambda x: dev.unary_bw("tanh", x, ys(), x, gs()))(xs()), 4 * big),
+            ("prelu_fw", lambda: dev.const_fw("prelu", xs(), 0.01), 2 * big),
+            ("add_fw", lambda: dev.binary_fw("add", xs(), ys()), 3 * big),
+            ("multiply_bw", lambda: (lambda x, y: dev.binary_bw("multiply", x, y, x, y, gs(), g2s()))(xs(), ys()), 7 * big),
+            ("bias_add_fw", lambda: dev.binary_fw("add", xbs(), bias), 2 * med + vol * item),
+            ("bias_add_bw", lambda: (lambda xb: dev.binary_bw("add", xb, bias, xb, xb, gxbs(), gbias))(xbs()),
+             3 * med + 2 * vol * item),
+            ("inplace_add", lambda: dev.inplace_add(xs(), ys()), 3 * big),
+            ("inplace_multiply_const", lambda: dev.inplace_multiply_const(1.0, ys()), 2 * big),
             ("bias_add_fw_2048x64", lambda: dev.binary_fw("add", sx, sbias), (2 * sv * sb + sv) * item),
             ("bias_add_bw_2048x64", lambda: dev.binary_bw("add", sx, sbias, sx, sx, sg, sgb),
              (3 * sv * sb + 2 * sv) * item),
@@ -428,27 +444,27 @@ def measure_pointwise(reps=20):
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
                   % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
                   file=sys.stderr, flush=True)
-        del x, y, g, g2, bias, gbias, xb, gxb, sbias, sx, sg, sgb, cases
+        del xs, ys, gs, g2s, bias, gbias, xbs, gxbs, sbias, sx, sg, sgb, cases
         # moving and reducing along a dimension: a 4096 x 4096 matrix with a minibatch of 4
         # (64 Mi elements) and the softmax of a 10000-word vocabulary over a minibatch of 64
         r, bs = 4096, 4
-        m = dev.new_tensor_by_constant(S([r, r], bs), 0.5)
-        gm = dev.new_tensor_by_constant(S([r, r], bs), 0.0)
+        ms = Ring(lambda: dev.new_tensor_by_constant(S([r, r], bs), 0.5))
+        gms = Ring(lambda: dev.new_tensor_by_constant(S([r, r], bs), 0.0))
         whole = r * r * bs * item
         logits = dev.new_tensor_by_constant(S([10000], 64), 0.5)
         table = dev.new_tensor_by_constant(S([650, 10000]), 0.5)
         gtable = dev.new_tensor_by_constant(S([650, 10000]), 0.0)
         ids = [(7919 * i) % 10000 for i in range(64)]
         picked = dev.pick_fw(table, ids, 1)
-        half = dev.slice_fw(m, 0, 0, r // 2)
+        halves = Ring(lambda: dev.slice_fw(ms(), 0, 0, r // 2))
         cases = [
-            ("slice_fw_rows", lambda: dev.slice_fw(m, 0, 0, r // 2), whole),
-            ("slice_bw_rows", lambda: dev.slice_bw(half, 0, 0, gm), whole // 2 * 3),
-            ("concat_fw_cols", lambda: dev.concat_fw([half, half], 1), whole * 2),
-            ("transpose_fw", lambda: dev.transpose_fw(m), 2 * whole),
-            ("sum_fw_dim0", lambda: dev.reduce_fw("sum", m, 0), whole + whole // r),
-            ("sum_fw_dim1", lambda: dev.reduce_fw("sum", m, 1), whole + whole // r),
-            ("max_fw_dim1", lambda: dev.reduce_fw("max", m, 1), whole + whole // r),
+            ("slice_fw_rows", lambda: dev.slice_fw(ms(), 0, 0, r // 2), whole),
+            ("slice_bw_rows", lambda: dev.slice_bw(halves(), 0, 0, gms()), whole // 2 * 3),
+            ("concat_fw_cols", lambda: dev.concat_fw([halves(), halves()], 1), whole * 2),
+            ("transpose_fw", lambda: dev.transpose_fw(ms()), 2 * whole),
+            ("sum_fw_dim0", lambda: dev.reduce_fw("sum", ms(), 0), whole + whole // r),
+            ("sum_fw_dim1", lambda: dev.reduce_fw("sum", ms(), 1), whole + whole // r),
+            ("max_fw_dim1", lambda: dev.reduce_fw("max", ms(), 1), whole + whole // r),
             ("logsumexp_fw_vocab", lambda: dev.reduce_fw("logsumexp", logits, 0), (640000 + 64) * item),
             ("broadcast_fw_vocab", lambda: dev.broadcast_fw(dev.reduce_fw("sum", logits, 0), 0, 10000),
              (2 * 640000 + 128) * item),
@@ -462,20 +478,20 @@ def measure_pointwise(reps=20):
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
                   % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
                   file=sys.stderr, flush=True)
-        del m, gm, logits, table, gtable, picked, half, cases
+        del ms, gms, logits, table, gtable, picked, halves, cases
         # random tensors (results written once) and copies between device objects on this GPU
         # (one read, one write; to the other storage width: converted on the way)
         n = 64 << 20
         other = pa.HIP16(0, storage="f16") if storage == "f32" else pa.HIP(0)
         other_item = 2 if storage == "f32" else 4
-        src = dev.new_tensor_by_constant(S([n]), 0.5)
+        srcs = Ring(lambda: dev.new_tensor_by_constant(S([n]), 0.5))
         cases = [
             ("random_uniform", lambda: dev.random_uniform(S([n]), -1.0, 1.0), n * item),
             ("random_normal", lambda: dev.random_normal(S([n]), 0.0, 1.0), n * item),
             ("random_bernoulli", lambda: dev.random_bernoulli(S([n]), 0.5), n * item),
-            ("copy_tensor_same_storage", lambda: dev.copy_tensor(src), 2 * n * item),
+            ("copy_tensor_same_storage", lambda: dev.copy_tensor(srcs()), 2 * n * item),
             # to another device object: the call drains both streams itself, so the host clock times it
-            ("copy_tensor_to_" + ("f16" if storage == "f32" else "f32"), lambda: other.copy_tensor(src),
+            ("copy_tensor_to_" + ("f16" if storage == "f32" else "f32"), lambda: other.copy_tensor(srcs()),
              n * (item + other_item)),
         ]
         for name, fn, nbytes in cases:
@@ -485,7 +501,7 @@ def measure_pointwise(reps=20):
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
                   % (name, storage, sec * 1e6, out[-1]["gbs"], 100 * out[-1]["frac_hbm_peak"]),
                   file=sys.stderr, flush=True)
-        del src, cases
+        del srcs, cases
         other.close()
         dev.close()
     return out
