@@ -11,6 +11,7 @@ workload (square batched fp32), `workloads` carries the same figures for all
 five.  The CPU figures come from the CPU oracle timed on this host.
 """
 import argparse
+import collections
 import copy
 import ctypes
 import json
@@ -349,13 +350,13 @@ def measure(name, steps, warmup, skip_cpu, deterministic=False, in_order=False, 
     return out
 
 
-def _event_seconds(dev, fn, reps):
+def _event_seconds(dev, fn, reps, warm=2):
     """Average seconds of one fn() over `reps` back-to-back calls, by events on the library's stream."""
     ctx = dev.ctx()
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     _lib.call("phip_event_create", ctx, ctypes.byref(e0))
     _lib.call("phip_event_create", ctx, ctypes.byref(e1))
-    for _ in range(2):
+    for _ in range(warm):
         fn()
     dev.sync()
     _lib.call("phip_event_record", ctx, e0)
@@ -369,9 +370,9 @@ def _event_seconds(dev, fn, reps):
     return ms.value * 1e-3 / reps
 
 
-def _wall_seconds(dev, fn, reps):
+def _wall_seconds(dev, fn, reps, warm=2):
     """Average seconds of one blocking fn() (a call that waits for the device itself) by the host clock."""
-    for _ in range(2):
+    for _ in range(warm):
         fn()
     dev.sync()
     t0 = time.perf_counter()
@@ -390,10 +391,18 @@ def measure_pointwise(reps=20):
     The large cases walk round several sets of operands, so that no call finds its operands in the 256 MB
     Infinity Cache from the call before: repeated over ONE set, a copy of 256 MiB reads 5.4 TB/s, the same copy
     with streaming stores 8.6 TB/s (the source then stays in the cache between calls), and one of 1 GiB 5.1
-    either way - the rate of HBM is what the rotation shows."""
+    either way - the rate of HBM is what the rotation shows.  Results rotate too: each case keeps its last
+    SETS results alive, so the memory pool hands a call the block of the oldest one and not the block the
+    call before has just written (a 128 MiB result written over and over stays in that cache: the 16-bit
+    transpose then reads 6.2 TB/s, with results of 256 MiB and more 5.2)."""
     S = pa.Shape
     out = []
     SETS = 4
+
+    def kept(fn):
+        """fn, with its last SETS results held."""
+        held = collections.deque(maxlen=SETS)
+        return lambda: held.append(fn())
 
     class Ring:
         """SETS tensors of one shape, handed out in turn."""
@@ -438,7 +447,7 @@ def measure_pointwise(reps=20):
              (3 * sv * sb + 2 * sv) * item),
         ]
         for name, fn, nbytes in cases:
-            sec = _event_seconds(dev, fn, reps)
+            sec = _event_seconds(dev, kept(fn), reps, warm=SETS + 2)
             out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
                         "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
@@ -472,7 +481,7 @@ def measure_pointwise(reps=20):
             ("pick_bw_embedding", lambda: dev.pick_bw(picked, ids, 1, gtable), 3 * 650 * 64 * item),
         ]
         for name, fn, nbytes in cases:
-            sec = _event_seconds(dev, fn, reps)
+            sec = _event_seconds(dev, kept(fn), reps, warm=SETS + 2)
             out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
                         "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"
@@ -495,7 +504,7 @@ def measure_pointwise(reps=20):
              n * (item + other_item)),
         ]
         for name, fn, nbytes in cases:
-            sec = (_wall_seconds if name.startswith("copy_tensor_to") else _event_seconds)(dev, fn, reps)
+            sec = (_wall_seconds if name.startswith("copy_tensor_to") else _event_seconds)(dev, kept(fn), reps, warm=SETS + 2)
             out.append({"kernel": name, "dtype": storage, "bytes": nbytes, "us": sec * 1e6,
                         "gbs": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / PEAK_HBM_GBS})
             print("# %-24s %s  %9.1f us  %7.0f GB/s (%.1f%% of HBM peak)"

@@ -5,6 +5,7 @@
 // gradient summed over the minibatch, repeated indices) one thread owns the
 // destination and adds the sources in order, so results do not depend on
 // scheduling and no atomics are used.
+#include <type_traits>
 #include <vector>
 
 #include "phip_pointwise.h"
@@ -195,6 +196,68 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T *src, T *dst,
   for (uint32_t u = 0; u < kTr / 4; ++u) {
     const uint32_t ii = ty + 4 * u, i = i0 + ii, j = j0 + tx;
     if (i < rows && j < cols) put<T, ACC>(dst + ofs + j + (size_t)i * cols, tile[tx][ii]);
+  }
+}
+
+// rows and cols even: the matrix is taken as 2 x 2 blocks. A lane reads one pair
+// of vertically adjacent elements (one word: 4 bytes of 16-bit storage, 8 of fp32)
+// from each of two neighbouring source columns (rows 2a, 2a+1 of columns 2b, 2b+1),
+// regroups the four elements into the two destination words (columns 2b, 2b+1 of
+// destination rows 2a and 2a+1), and the blocks of a tile then move through LDS as
+// whole words, one plane per destination-row parity. A wavefront reads 64 words
+// in a row; a tile is 64 blocks along the source rows by kTb along its columns
+// (32 KiB of source either way), so a thread has 32 KiB / 256 in flight before
+// the first LDS write, twice what the one-element form holds.
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kBlock) void transpose_pairs_kernel(const T *src, T *dst, uint32_t rows, uint32_t cols) {
+  typedef typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type Word;
+  constexpr uint32_t kHalf = 8 * sizeof(T);             // bits per element
+  constexpr Word kLow = (Word(1) << kHalf) - 1;
+  constexpr uint32_t kTb = sizeof(T) == 2 ? 64 : 32;    // blocks of a tile along the source columns
+  constexpr uint32_t kRw = 64 / kTb;                    // destination rows a wavefront writes per access
+  __shared__ Word tile[2][kTb][kTr + 1];
+  const size_t ofs = (size_t)blockIdx.z * rows * cols;
+  const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const uint32_t a0 = blockIdx.x * kTr, b0 = blockIdx.y * kTb;  // in 2 x 2 blocks
+  const uint32_t ra = rows / 2, cb = cols / 2;
+  const Word *sw = reinterpret_cast<const Word *>(src + ofs);
+  Word w0[kTb / 4], w1[kTb / 4];
+#pragma unroll
+  for (uint32_t u = 0; u < kTb / 4; ++u) {
+    const uint32_t a = a0 + tx, b = b0 + ty + 4 * u;
+    const bool in = a < ra && b < cb;
+    w0[u] = in ? sw[a + (size_t)(2 * b) * ra] : Word(0);
+    w1[u] = in ? sw[a + (size_t)(2 * b + 1) * ra] : Word(0);
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kTb / 4; ++u) {
+    tile[0][ty + 4 * u][tx] = (w0[u] & kLow) | (w1[u] << kHalf);
+    tile[1][ty + 4 * u][tx] = (w0[u] >> kHalf) | (w1[u] & ~kLow);
+  }
+  __syncthreads();
+  Word *dw = reinterpret_cast<Word *>(dst + ofs);
+  const uint32_t bl = tx % kTb, ah = tx / kTb;
+#pragma unroll
+  for (uint32_t u = 0; u < kTr / (4 * kRw); ++u) {
+    const uint32_t aa = ty * kRw + ah + 4 * kRw * u, a = a0 + aa, b = b0 + bl;
+    if (a < ra && b < cb) {
+#pragma unroll
+      for (uint32_t par = 0; par < 2; ++par) {
+        Word *q = dw + b + (size_t)(2 * a + par) * cb;
+        Word w = tile[par][bl][aa];
+        if constexpr (ACC) {
+          struct Two {
+            T e[2];
+          };
+          const Two old = __builtin_bit_cast(Two, *q), add = __builtin_bit_cast(Two, w);
+          Two r;
+          r.e[0] = from_f32<T>(to_f32(old.e[0]) + to_f32(add.e[0]));
+          r.e[1] = from_f32<T>(to_f32(old.e[1]) + to_f32(add.e[1]));
+          w = __builtin_bit_cast(Word, r);
+        }
+        *q = w;
+      }
+    }
   }
 }
 
@@ -392,6 +455,22 @@ int transpose(phip_ctx *ctx, bool accumulate, const void *src, void *dst, uint32
   if (rows == 0 || cols == 0 || bs == 0) return PHIP_OK;
   PHIP_REQUIRE(src != nullptr && dst != nullptr, "null pointer");
   PHIP_REQUIRE(bs <= 65535u && (cols + kTr - 1) / kTr <= 65535u, "shape exceeds what one launch covers");
+  {
+    constexpr uint32_t kTb = sizeof(T) == 2 ? 64 : 32;
+    if (rows % 2 == 0 && cols % 2 == 0 && reinterpret_cast<uintptr_t>(src) % (2 * sizeof(T)) == 0 &&
+        reinterpret_cast<uintptr_t>(dst) % (2 * sizeof(T)) == 0 && (cols / 2 + kTb - 1) / kTb <= 65535u) {
+      const dim3 pairs((rows / 2 + kTr - 1) / kTr, (cols / 2 + kTb - 1) / kTb, bs);
+      if (accumulate) {
+        hipLaunchKernelGGL((transpose_pairs_kernel<T, true>), pairs, dim3(kBlock), 0, ctx->stream,
+                           static_cast<const T *>(src), static_cast<T *>(dst), rows, cols);
+      } else {
+        hipLaunchKernelGGL((transpose_pairs_kernel<T, false>), pairs, dim3(kBlock), 0, ctx->stream,
+                           static_cast<const T *>(src), static_cast<T *>(dst), rows, cols);
+      }
+      PHIP_LAUNCH_CHECK();
+      return PHIP_OK;
+    }
+  }
   const dim3 grid((rows + kTr - 1) / kTr, (cols + kTr - 1) / kTr, bs);
   if (accumulate) {
     hipLaunchKernelGGL((transpose_kernel<T, true>), grid, dim3(kBlock), 0, ctx->stream, static_cast<const T *>(src),

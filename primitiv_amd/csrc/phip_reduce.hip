@@ -81,6 +81,22 @@ struct ExtremumOp {
   __device__ static float result(const State &a) { return SIGN > 0 ? a.v : -a.v; }
 };
 
+// Extremum alone, for a launch that writes values: the same comparisons as
+// ExtremumOp (a NaN never enters, the first of equal values stays) without the
+// index, at a third of the instructions per element and half the state.  (Of a
+// +0 and a -0, which compare equal, the one returned need not be the first.)
+template <int SIGN>
+struct ExtremumValueOp {
+  struct State { float v; };
+  __device__ static State init() { return {-kInf}; }
+  __device__ static void push(State &a, float v, uint32_t) {
+    const float w = SIGN > 0 ? v : -v;
+    a.v = w > a.v ? w : a.v;
+  }
+  __device__ static void merge(State &a, const State &b) { a.v = b.v > a.v ? b.v : a.v; }
+  __device__ static float result(const State &a) { return SIGN > 0 ? a.v : -a.v; }
+};
+
 // What a launch writes per output element.
 enum class Emit { Value, Index, Gradient };
 
@@ -143,20 +159,124 @@ __device__ inline typename OP::State walk(const T *p, size_t stride_elems, uint3
   return st[0];
 }
 
+// A contiguous run of n elements (n a multiple of V, p aligned to V elements)
+// taken V elements per access: lane `first` of `step` takes packs first,
+// first + step, ...; U packs are in flight together.
+template <typename T, typename OP, int V, int U = 4>
+__device__ inline typename OP::State walk_packs(const T *p, uint32_t first, uint32_t step, uint32_t n) {
+  struct alignas(V * sizeof(T)) Pack {
+    T c[V];
+  };
+  const Pack *q = reinterpret_cast<const Pack *>(p);
+  const uint32_t end = n / V;
+  typename OP::State st[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) st[u] = OP::init();
+  uint32_t j = first;
+  for (; j < end && end - j > (U - 1) * step; j += U * step) {
+    Pack v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = q[j + u * step];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < V; ++k) OP::push(st[u], to_f32(v[u].c[k]), (j + u * step) * V + k);
+  }
+#pragma unroll
+  for (int u = 0; u < U - 1; ++u) {
+    if (j < end) {
+      const Pack v = q[j];
+#pragma unroll
+      for (int k = 0; k < V; ++k) OP::push(st[u], to_f32(v.c[k]), j * V + k);
+    }
+    j += step;
+  }
+#pragma unroll
+  for (int w = 1; w < U; w *= 2) {
+#pragma unroll
+    for (int u = 0; u + w < U; u += 2 * w) OP::merge(st[u], st[u + w]);
+  }
+  return st[0];
+}
+
 // A long reduction may be cut into `splits` ranges of `chunk` positions, each
-// reduced by its own workgroup into partial[(o*splits + sp)*base + i]; a second
-// launch (reduce_finish_kernel) merges the ranges in order.  splits == 1 writes
-// the result directly.
+// reduced by its own workgroup into partial[(o*splits + sp)*base + i]. The
+// workgroup that finishes last of a group's ranges (a counter per group tells)
+// merges them in order and writes the results; without counters a second
+// launch (reduce_finish_kernel) does.  splits == 1 writes the result directly.
 struct Split {
   uint32_t splits, chunk;
+  uint32_t *tickets;   // splits > 1: one zeroed counter per group of outputs, left zeroed; or null
 };
+
+// Partial states travel between workgroups, which may sit on different L2s:
+// device-scope accesses, word by word, go past those caches.
+template <typename State>
+__device__ inline void store_state(State *p, const State &st) {
+  uint32_t w[sizeof(State) / 4];
+  __builtin_memcpy(w, &st, sizeof(State));
+#pragma unroll
+  for (unsigned k = 0; k < sizeof(State) / 4; ++k)
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p) + k, w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename State>
+__device__ inline State load_state(const State *p) {
+  uint32_t w[sizeof(State) / 4];
+#pragma unroll
+  for (unsigned k = 0; k < sizeof(State) / 4; ++k)
+    w[k] = __hip_atomic_load(reinterpret_cast<const uint32_t *>(p) + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  State st;
+  __builtin_memcpy(&st, w, sizeof(State));
+  return st;
+}
+
+// Called by all threads of a workgroup after its partial states were stored:
+// true in the workgroup that is the last of the group's `splits` to get here.
+// Each lane waits until memory has acknowledged its own stores, the barrier puts
+// all of them before thread 0's ticket, and the ticket is a device-scope atomic
+// on one address, so the one who draws the last ticket does so after every other
+// workgroup's stores arrived. The counter is left zeroed for the next launch.
+__device__ inline bool last_of_group(uint32_t *ticket, uint32_t splits, uint32_t *flag) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = drawn == splits - 1u;
+    if (last) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last ? 1u : 0u;
+  }
+  __syncthreads();
+  return *flag != 0;
+}
+
+// The ranges of one output merged in order.
+template <typename T, typename OP, Emit EMIT>
+__device__ inline void merge_ranges(const typename OP::State *partial, uint32_t splits, T *y, uint32_t *index_out,
+                                    const T *gy, T *gx, size_t o, uint32_t i, uint32_t base, uint32_t n) {
+  // eight loads in flight at a time: one after the other they would cost a trip to memory each
+  typename OP::State st = OP::init();
+  for (uint32_t r0 = 0; r0 < splits; r0 += 8) {
+    typename OP::State v[8];
+#pragma unroll
+    for (uint32_t u = 0; u < 8; ++u)
+      v[u] = load_state(partial + (o * splits + (r0 + u < splits ? r0 + u : splits - 1)) * base + i);
+#pragma unroll
+    for (uint32_t u = 0; u < 8; ++u)
+      if (r0 + u < splits) {
+        if (r0 + u == 0) st = v[0];
+        else OP::merge(st, v[u]);
+      }
+  }
+  emit<T, OP, EMIT>(st, y, index_out, gy, gx, o * base + i, o * n * base + i, base, n);
+}
 
 template <typename T, typename OP, Emit EMIT>
 __device__ inline void finish(const typename OP::State &st, typename OP::State *partial, Split sp, uint32_t r,
                               T *y, uint32_t *index_out, const T *gy, T *gx, size_t o, uint32_t i, uint32_t base,
                               uint32_t n) {
   if (sp.splits > 1) {
-    partial[(o * sp.splits + r) * base + i] = st;
+    store_state(partial + (o * sp.splits + r) * base + i, st);
   } else {
     emit<T, OP, EMIT>(st, y, index_out, gy, gx, o * base + i, o * n * base + i, base, n);
   }
@@ -168,6 +288,7 @@ __global__ __launch_bounds__(kBlock) void reduce_block_kernel(const T *x, T *y, 
                                                                T *gx, typename OP::State *partial, Split sp,
                                                                uint32_t base, uint32_t n, size_t outputs) {
   __shared__ typename OP::State part[kBlock];
+  __shared__ uint32_t last;
   for (size_t b = blockIdx.x; b < outputs * sp.splits; b += gridDim.x) {
     const size_t q = b / sp.splits;
     const uint32_t r = (uint32_t)(b - q * sp.splits);
@@ -181,20 +302,28 @@ __global__ __launch_bounds__(kBlock) void reduce_block_kernel(const T *x, T *y, 
       __syncthreads();
     }
     if (threadIdx.x == 0) finish<T, OP, EMIT>(part[0], partial, sp, r, y, index_out, gy, gx, o, i, base, n);
+    if (sp.splits > 1 && sp.tickets != nullptr) {
+      if (last_of_group(sp.tickets + q, sp.splits, &last) && threadIdx.x == 0)
+        merge_ranges<T, OP, EMIT>(partial, sp.splits, y, index_out, gy, gx, o, i, base, n);
+    }
     __syncthreads();
   }
 }
 
 // base == 1: wavefront w of the grid owns outputs w, w + waves, ...; its lanes
 // stride along the contiguous run.
-template <typename T, typename OP, Emit EMIT>
+// V > 1: n is a multiple of V and x is aligned to V elements; a lane then takes V
+// neighbouring elements per access.
+template <typename T, typename OP, Emit EMIT, int V>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const T *x, T *y, uint32_t *index_out, const T *gy,
                                                               T *gx, uint32_t n, size_t outputs) {
   const uint32_t lane = threadIdx.x & 63;
   const size_t waves = (size_t)gridDim.x * (kBlock / 64);
   for (size_t q = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); q < outputs; q += waves) {
     const size_t first = q * n;
-    typename OP::State st = walk<T, OP>(x + first, 1, lane, 64, n);
+    typename OP::State st;
+    if constexpr (V > 1) st = walk_packs<T, OP, V>(x + first, lane, 64, n);
+    else st = walk<T, OP>(x + first, 1, lane, 64, n);
 #pragma unroll
     for (int w = 32; w > 0; w >>= 1) {
       typename OP::State other;
@@ -265,6 +394,7 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, 
                                                                uint32_t base, uint32_t n, uint32_t outer) {
   constexpr int TY = kBlock / TX;
   __shared__ typename OP::State part[TY][TX][V];
+  __shared__ uint32_t last;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const uint32_t per_o = (base + TX * V - 1) / (TX * V);
   for (size_t b = blockIdx.x; b < (size_t)per_o * outer * sp.splits; b += gridDim.x) {
@@ -285,6 +415,13 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, 
       for (int k = 0; k < V; ++k) {
         for (int u = 1; u < TY; ++u) OP::merge(st[k], part[u][tx][k]);
         finish<T, OP, EMIT>(st[k], partial, sp, r, y, index_out, gy, gx, o, i + k, base, n);
+      }
+    }
+    if (sp.splits > 1 && sp.tickets != nullptr) {
+      if (last_of_group(sp.tickets + t, sp.splits, &last)) {
+        const uint32_t i0 = (uint32_t)(t - o * per_o) * TX * V;
+        for (uint32_t e = threadIdx.x; e < TX * V && i0 + e < base; e += kBlock)
+          merge_ranges<T, OP, EMIT>(partial, sp.splits, y, index_out, gy, gx, o, i0 + e, base, n);
       }
     }
     __syncthreads();
@@ -308,7 +445,7 @@ __global__ __launch_bounds__(kBlock) void reduce_finish_kernel(const typename OP
 // How many ranges to cut n into so that `groups` workgroups become about four
 // per compute unit, each range at least `min_chunk` long.
 inline Split choose_split(size_t groups, uint32_t n, uint32_t min_chunk, size_t cus) {
-  Split sp = {1, n};
+  Split sp = {1, n, nullptr};
   const size_t want = 4 * cus;
   if (groups >= want || n < 2 * min_chunk) return sp;
   size_t splits = (want + groups - 1) / groups;
@@ -333,8 +470,15 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
   if (!by_block && !by_tiles) {
     if (by_rows) {
       const size_t blocks = (outputs + kBlock / 64 - 1) / (kBlock / 64);
-      hipLaunchKernelGGL((reduce_rows_kernel<T, OP, EMIT>), dim3((unsigned)(blocks < cap ? blocks : cap)),
-                         dim3(kBlock), 0, ctx->stream, x, y, index_out, gy, gx, n, outputs);
+      constexpr int kPack = 16 / sizeof(T);   // 16 bytes per lane and access
+      const dim3 rows_grid((unsigned)(blocks < cap ? blocks : cap));
+      if (n % kPack == 0 && n >= 64 * kPack && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        hipLaunchKernelGGL((reduce_rows_kernel<T, OP, EMIT, kPack>), rows_grid, dim3(kBlock), 0, ctx->stream, x, y,
+                           index_out, gy, gx, n, outputs);
+      } else {
+        hipLaunchKernelGGL((reduce_rows_kernel<T, OP, EMIT, 1>), rows_grid, dim3(kBlock), 0, ctx->stream, x, y,
+                           index_out, gy, gx, n, outputs);
+      }
     } else {
       hipLaunchKernelGGL((reduce_column_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
                          ctx->stream, x, y, index_out, gy, gx, base, n, outputs);
@@ -342,16 +486,21 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
     PHIP_LAUNCH_CHECK();
     return PHIP_OK;
   }
-  // 16-bit storage: two columns per lane (4-byte accesses) when base and the address allow
-  constexpr int kCols = sizeof(T) == 2 ? 2 : 1;
-  const bool wide = kCols > 1 && base >= 128 && base % kCols == 0 && reinterpret_cast<uintptr_t>(x) % (kCols * sizeof(T)) == 0;
+  // 8 bytes per lane and access (two fp32 or four 16-bit columns) when base and the address allow,
+  // else 4 bytes for 16-bit storage (two columns)
+  constexpr int kCols = 8 / sizeof(T), kHalf = sizeof(T) == 2 ? 2 : 1;
+  const bool wide = base >= 64 * kCols && base % kCols == 0 && reinterpret_cast<uintptr_t>(x) % 8 == 0;
+  const bool wide2 = !wide && kHalf > 1 && base >= 64 * kHalf && base % kHalf == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0;
   const int tx = base >= 64 ? 64 : 16;
-  const size_t groups = by_block ? outputs : (size_t)((base + tx * (wide ? kCols : 1) - 1) / (tx * (wide ? kCols : 1))) * outer;
-  const Split sp = choose_split(groups, n, by_block ? 8192 : 256, cus);
+  const int cols = wide ? kCols : wide2 ? kHalf : 1;
+  const size_t groups = by_block ? outputs : (size_t)((base + tx * cols - 1) / (tx * cols)) * outer;
+  Split sp = choose_split(groups, n, by_block ? 1024 : 256, cus);
   void *block = nullptr;
   if (sp.splits > 1) {
     const int rc = phip_pool_alloc(ctx, sizeof(State) * outputs * sp.splits, &block, nullptr);
     if (rc != PHIP_OK) return rc;
+    // the last workgroup of a group merges its ranges when there is a counter per group; else a second launch does
+    if (groups <= (size_t)kTicketSlots) sp.tickets = ctx->tile_tickets;
   }
   State *partial = static_cast<State *>(block);
   const size_t blocks = groups * sp.splits;
@@ -362,6 +511,9 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
   } else if (wide) {
     hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64, kCols>), grid, dim3(kBlock), 0, ctx->stream, x, y,
                        index_out, gy, gx, partial, sp, base, n, outer);
+  } else if (wide2) {
+    hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64, kHalf>), grid, dim3(kBlock), 0, ctx->stream, x, y,
+                       index_out, gy, gx, partial, sp, base, n, outer);
   } else if (tx == 64) {
     hipLaunchKernelGGL((reduce_tiles_kernel<T, OP, EMIT, 64, 1>), grid, dim3(kBlock), 0, ctx->stream, x, y, index_out,
                        gy, gx, partial, sp, base, n, outer);
@@ -370,8 +522,10 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
                        gy, gx, partial, sp, base, n, outer);
   }
   if (sp.splits > 1) {
-    hipLaunchKernelGGL((reduce_finish_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
-                       ctx->stream, partial, sp.splits, y, index_out, gy, gx, base, n, outputs);
+    if (sp.tickets == nullptr) {
+      hipLaunchKernelGGL((reduce_finish_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
+                         ctx->stream, partial, sp.splits, y, index_out, gy, gx, base, n, outputs);
+    }
     phip_pool_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
   }
   PHIP_LAUNCH_CHECK();
@@ -392,9 +546,9 @@ int reduce_fw(phip_ctx *ctx, int op, const void *x, void *y, uint32_t base, uint
     case PHIP_LOGSUMEXP:
       return launch_reduce<T, LogSumExpOp, Emit::Value>(ctx, px, py, nullptr, nullptr, nullptr, base, n, outer);
     case PHIP_MAX:
-      return launch_reduce<T, ExtremumOp<1>, Emit::Value>(ctx, px, py, nullptr, nullptr, nullptr, base, n, outer);
+      return launch_reduce<T, ExtremumValueOp<1>, Emit::Value>(ctx, px, py, nullptr, nullptr, nullptr, base, n, outer);
     default:
-      return launch_reduce<T, ExtremumOp<-1>, Emit::Value>(ctx, px, py, nullptr, nullptr, nullptr, base, n, outer);
+      return launch_reduce<T, ExtremumValueOp<-1>, Emit::Value>(ctx, px, py, nullptr, nullptr, nullptr, base, n, outer);
   }
 }
 

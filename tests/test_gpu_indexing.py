@@ -189,7 +189,11 @@ def test_dimension_ops_match_oracle(dev, dims, batch):
 # One shape per launch shape of the reduction (wavefront per contiguous run, lanes
 # along base with n split, workgroup per output, thread per output), ragged sizes.
 REDUCE_SHAPES = [([100, 300], 2, 0), ([33, 1031], 1, 0), ([70, 100], 3, 1), ([129, 517], 2, 1), ([20, 50], 40, 1),
-                 ([17, 1000, 3], 1, 1), ([5000], 3, 0), ([20011], 2, 0), ([3, 9000], 2, 1), ([40, 20], 30, 0), ([4, 64, 2], 5, 1)]
+                 ([17, 1000, 3], 1, 1), ([5000], 3, 0), ([20011], 2, 0), ([3, 9000], 2, 1), ([40, 20], 30, 0), ([4, 64, 2], 5, 1),
+                 # a contiguous run taken 16 bytes per lane (length a multiple of 4, at least 256, many outputs)
+                 ([256, 520], 1, 0), ([260, 300], 2, 0), ([1028, 530], 1, 0),
+                 # two columns per lane (even stride of at least 128 below the reduced dimension)
+                 ([128, 517], 2, 1), ([130, 300], 2, 1), ([386, 40, 3], 1, 1)]
 
 
 @pytest.mark.parametrize("dims,batch,dim", REDUCE_SHAPES)
@@ -217,7 +221,8 @@ def test_reduction_launch_shapes_match_oracle(dev, dims, batch, dim):
             assert np.allclose(gx.to_vector(), oracle.extremum_bw(x, yv, gyv, g0, dims, batch, dim), atol=1e-6)
 
 
-@pytest.mark.parametrize("d1,d2,bs", [(1, 1, 1), (5, 7, 3), (64, 32, 2), (100, 257, 4), (1000, 33, 1)])
+@pytest.mark.parametrize("d1,d2,bs", [(1, 1, 1), (5, 7, 3), (64, 32, 2), (100, 257, 4), (1000, 33, 1), (130, 258, 2), (256, 66, 3),
+                                      (2, 2, 1), (2, 1000, 2)])
 def test_transpose_and_batch_ops_match_oracle(dev, d1, d2, bs):
     rng = np.random.default_rng(d1 + d2)
     x = rng.standard_normal(d1 * d2 * bs).astype(np.float32)
@@ -331,6 +336,24 @@ def test_half_storage_matches_oracle(dev16):
     assert np.array_equal(dev16.batch_pick_fw(tx, [2, 2, 0]).to_vector(), oracle.batch_pick_fw(xr, 1200, [2, 2, 0]))
 
 
+@pytest.mark.parametrize("d1,d2,bs", [(2, 2, 1), (40, 30, 3), (130, 258, 2), (128, 128, 1), (256, 66, 3), (41, 30, 2),
+                                      (40, 31, 2), (1, 64, 1)])
+def test_half_storage_transpose(dev16, d1, d2, bs):
+    # even extents move as 2 x 2 blocks of elements (tiles of 128 x 128 elements of 16-bit storage), odd ones one element per lane
+    rng = np.random.default_rng(d1 * 1000 + d2)
+    x = rng.standard_normal(d1 * d2 * bs).astype(np.float32)
+    tx = dev16.new_tensor_by_vector(S([d1, d2], bs), x)
+    xr = tx.to_vector()
+    y = dev16.transpose_fw(tx)
+    assert y.shape() == S([d2, d1], bs)
+    assert np.array_equal(y.to_vector(), oracle.transpose_fw(xr, d1, d2, bs))
+    g0 = round_to_storage(rng.standard_normal(x.size).astype(np.float32), dev16._SUFFIX)
+    gx = dev16.new_tensor_by_vector(S([d1, d2], bs), g0)
+    dev16.transpose_bw(tx, y, y, gx)                    # gx += transpose(gy), rounded once per element
+    want = round_to_storage(oracle.transpose_bw(y.to_vector(), g0, d1, d2, bs), dev16._SUFFIX)
+    assert np.array_equal(gx.to_vector(), want)
+
+
 def _aligned_copies(dev, exact_sum):
     # extents and offsets that are multiples of 16 bytes in every storage type: the
     # copies then move whole 16-byte packs
@@ -366,11 +389,14 @@ def test_half_storage_aligned_copies_match_oracle(dev16):
     _aligned_copies(dev16, False)
 
 
-@pytest.mark.parametrize("dims,batch,dim", [([130, 517], 2, 1), ([256, 40, 3], 1, 1), ([129, 300], 1, 1), ([64, 1031], 3, 0)])
+@pytest.mark.parametrize("dims,batch,dim", [([130, 517], 2, 1), ([256, 40, 3], 1, 1), ([129, 300], 1, 1), ([64, 1031], 3, 0),
+                                            ([260, 300], 2, 1), ([516, 70, 2], 1, 1), ([512, 520], 1, 0), ([520, 300], 2, 0),
+                                            ([1032, 515], 1, 0)])
 def test_half_storage_reduction_launch_shapes(dev16, dims, batch, dim):
-    # 16-bit storage reduces two columns per lane when the stride below the reduced
-    # dimension is even and at least 128 (first two shapes); odd and short strides and
-    # a leading-dimension reduction take the other launch shapes
+    # 16-bit storage reduces four columns per lane when the stride below the reduced
+    # dimension is a multiple of 4 and at least 256, two when it is even and at least
+    # 128; odd and short strides take one. A leading-dimension reduction walks each
+    # run 8 elements per lane when its length is a multiple of 8 and at least 512.
     rng = np.random.default_rng(dims[0] + batch)
     n = int(np.prod(dims)) * batch
     for x in (rng.standard_normal(n).astype(np.float32), rng.integers(-3, 4, n).astype(np.float32)):
