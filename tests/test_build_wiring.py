@@ -1,4 +1,5 @@
-"""The PRIMITIV_USE_HIP build wiring: the seven edits that INTEGRATION.md asks a maintainer to make
+"""The PRIMITIV_USE_HIP build wiring: the edits a maintainer makes to primitiv's tree to add the backend
+(sources copied in, the CMake option, the two CMake fragments included, the config macro, the umbrella headers)
 are applied to a scratch copy of primitiv, the copy is configured with the option on and built
 (hipcc cross-compiles gfx950 without a GPU), and a C program against the three libraries asks the C
 API for a HIP device.  Skipped where the primitiv source tree is absent (any GPU box)."""
@@ -40,7 +41,7 @@ def _insert(path, anchor, text, before=False, occurrence=1):
 
 
 def apply_integration_edits(tree):
-    """INTEGRATION.md section 1, edits 1 - 6 (7 concerns the reference's gtest suite)."""
+    """The six edits that add the backend to a copy of primitiv's tree (a seventh, adding the backend to its gtest suite, is not needed here)."""
     # 1. the host side next to the other backends
     shutil.copytree(os.path.join(BACKEND, "primitiv", "devices", "hip"), os.path.join(tree, "primitiv", "devices", "hip"))
     shutil.copytree(os.path.join(BACKEND, "primitiv", "c", "devices", "hip"),
