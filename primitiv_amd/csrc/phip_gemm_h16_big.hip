@@ -371,7 +371,10 @@ struct FragReader {
   }
 };
 
-template <bool A_KMAJOR, bool B_KMAJOR, bool BF16, int WB>
+// NS: LDS stages (K tiles resident or on their way).  Two is what two workgroups per CU (128 x 128 tiles) or one
+// (256 x 256) leave room for; a launch of 128 x 128 tiles with at most one workgroup per CU takes four, so that
+// three K tiles are in flight where the loop otherwise waits for its loads at every barrier.
+template <bool A_KMAJOR, bool B_KMAJOR, bool BF16, int WB, int NS = 2>
 __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel(const BigArgs g) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
   constexpr int BM = kTile<WB>, BN = kTile<WB>;
@@ -471,26 +474,35 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
     else lb.issue(rs_b, lds_run, q - NI, so_b);
   };
 
+  // Loads return in the order of issue: a tile has landed once at most the loads of the tiles issued after it
+  // (2 NI per tile and wavefront) are outstanding.
+  auto wait_for_tile = [&](int later_tiles) {
+    static_assert(NS <= 4 && (NS - 1) * 2 * NI <= 48, "wait counts are spelled out up to three tiles");
+    if (later_tiles <= 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else if (later_tiles == 1 && NI == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else if (later_tiles == 1) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    else if (later_tiles == 2 && NI == 4) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    else if (later_tiles == 2) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+    else if (NI == 4) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(48) lgkmcnt(0)" ::: "memory");
+  };
   describe_range();
   describe_tile();
   select_offsets();
 #pragma unroll
   for (int q = 0; q < 2 * NI; ++q) issue(q, 0);
-  if (kt_end > 1) {
-    next_tile();
-    describe_range();
-    describe_tile();
-    select_offsets();
 #pragma unroll
-    for (int q = 0; q < 2 * NI; ++q) issue(q, 1);
+  for (int st = 1; st < NS; ++st) {
+    if (kt_end > st) {
+      next_tile();
+      describe_range();
+      describe_tile();
+      select_offsets();
+#pragma unroll
+      for (int q = 0; q < 2 * NI; ++q) issue(q, st);
+    }
   }
-  // tile 0 has landed once all but the newest 2 NI loads (if tile 1 exists) are done
-  if (kt_end > 1) {
-    if constexpr (WB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
+  wait_for_tile((kt_end < NS ? kt_end : NS) - 1);
   __syncthreads();
 
   // The fragments of the two k steps of a tile live in two register buffers and
@@ -516,12 +528,12 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   for (int q = 0; q < 2 * NBK; ++q) read_frag(0, q, 0);
 
   static_assert(WB == 2 || NB >= 3 * 2 * NBK, "every third slot holds a read");
-  uint32_t flip_by = (uint32_t)kStage2Bytes;  // to the other stage and back
+  uint32_t flip_by = (uint32_t)kStage2Bytes;  // on to the next stage, or from the last back to the first
+  int stage = 0;                              // the stage that holds the tile being multiplied
   settle_matrix_pipe();  // the zeroed accumulators
-  // one K tile; LOADS: K tile kt + 2 exists and is fetched
+  // one K tile; LOADS: K tile kt + NS exists and is fetched into the stage this tile leaves
   auto tile = [&](auto loads_tag, int kt) {
     constexpr bool loads = decltype(loads_tag)::value;
-    const int stage = kt & 1;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -578,17 +590,25 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
         __builtin_amdgcn_sched_barrier(0);
       }
       if (t == 0) {
-        // own loads of tile kt+1 have landed, own reads of this stage are done;
-        // behind the barrier that holds for every wave
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        // own loads of tile kt+1 have landed (the tiles behind it may still be on their way), own
+        // reads of this stage are done; behind the barrier that holds for every wave
+        if constexpr (NS == 2) {
+          wait_for_tile(0);
+        } else if constexpr (loads) {
+          wait_for_tile(NS - 2);
+        } else {
+          const int later = kt_end - kt - 2;
+          wait_for_tile(later < NS - 2 ? later : NS - 2);
+        }
         __syncthreads();
       } else {
-        flip_by = 0u - flip_by;
+        stage = stage + 1 == NS ? 0 : stage + 1;
+        flip_by = stage == NS - 1 ? 0u - (uint32_t)((NS - 1) * kStage2Bytes) : (uint32_t)kStage2Bytes;
       }
     }
   };
   int kt = 0;
-  for (; kt + 2 < kt_end; ++kt) tile(std::true_type{}, kt);
+  for (; kt + NS < kt_end; ++kt) tile(std::true_type{}, kt);
   for (; kt < kt_end; ++kt) tile(std::false_type{}, kt);
   // every wave must be done with the stages before LDS is reused below
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -609,17 +629,18 @@ __global__ __launch_bounds__(kThreads, WB == 4 ? 1 : 2) void gemm_h16_lds_kernel
   }
 }
 
-template <bool BF16, int WB>
+template <bool BF16, int WB, int NS = 2>
 int launch_big(phip_ctx *ctx, const Gemm &p, const BigArgs &a) {
   const long grid = (long)a.tiles_m * a.tiles_n * p.batch;
-  constexpr int kFirstSlot = WB == 4 ? kSlotGemmH16Big : kSlotGemmH16Mid;
+  constexpr int kFirstSlot = NS > 2 ? kSlotGemmH16MidDeep : WB == 4 ? kSlotGemmH16Big : kSlotGemmH16Mid;
+  constexpr int kBytes = NS * kStage<WB>;
 #define PHIP_LDS(SLOT, AK, BKM)                                                                   \
   do {                                                                                            \
-    auto kern = gemm_h16_lds_kernel<AK, BKM, BF16, WB>;                                           \
+    auto kern = gemm_h16_lds_kernel<AK, BKM, BF16, WB, NS>;                                       \
     const int rc = raise_lds_limit(ctx, kFirstSlot + (SLOT) + (BF16 ? 3 : 0),                     \
-                                   reinterpret_cast<const void *>(kern), kLds<WB>);               \
+                                   reinterpret_cast<const void *>(kern), kBytes);                 \
     if (rc != PHIP_OK) return rc;                                                                 \
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kLds<WB>, ctx->stream, a);     \
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kThreads), kBytes, ctx->stream, a);       \
   } while (0)
   if (!p.a_kmajor && p.b_kmajor) PHIP_LDS(0, false, true);
   else if (!p.a_kmajor && !p.b_kmajor) PHIP_LDS(1, false, false);
@@ -675,9 +696,12 @@ int gemm_h16_big(phip_ctx *ctx, const Gemm &p, Elem elem, bool *handled) {
   a.accumulate = p.accumulate ? 1 : 0;
   a.a_bytes = (uint32_t)a_bytes;
   a.b_bytes = (uint32_t)b_bytes;
-  note_kernel(ctx, side == kTile<4> ? "h16_lds256" : "h16_lds128");
+  // 128 x 128 tiles, at most one per CU: four stages (128 KiB), three K tiles in flight
+  const bool deep = side == kTile<2> && tiles <= cus && a.total_ktiles >= 4;
+  note_kernel(ctx, side == kTile<4> ? "h16_lds256" : deep ? "h16_lds128_deep" : "h16_lds128");
   *handled = true;
   if (side == kTile<4>) return elem == Elem::BF16 ? launch_big<true, 4>(ctx, p, a) : launch_big<false, 4>(ctx, p, a);
+  if (deep) return elem == Elem::BF16 ? launch_big<true, 2, 4>(ctx, p, a) : launch_big<false, 2, 4>(ctx, p, a);
   return elem == Elem::BF16 ? launch_big<true, 2>(ctx, p, a) : launch_big<false, 2>(ctx, p, a);
 }
 

@@ -247,6 +247,7 @@ enum LdsSlot {
   kSlotGemmH16Skinny = 29,  // 8
   kSlotGemmF32LdsMixed = 37,  // 3
   kSlotGemmF32Lds64w = 40,    // 3
+  kSlotGemmH16MidDeep = 43,   // 6
 };
 
 // Allows `kernel` to use `bytes` of dynamic LDS (above the 64 KiB default) on

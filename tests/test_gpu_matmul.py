@@ -553,6 +553,12 @@ BIG_H16 = [  # di, dj, dk, ba, bb
     (1480, 1608, 1544, 1, 1),
     (520, 392, 264, 12, 12),
     (1288, 1032, 40, 1, 40),
+    # at most one such tile per CU: four K tiles resident or in flight; K of exactly 4 tiles, 5 with a tail
+    # of 8, 3 (the two-stage form), and a long one
+    (1032, 256, 776, 1, 1),
+    (1024, 264, 1024, 1, 1),
+    (1032, 192, 776, 1, 1),
+    (776, 3080, 760, 1, 1),
     # one large shared a against at least 16 Ki columns: the forward product runs on a transposed copy of a
     # (both operands then contiguous along k); ragged in every dimension, K tail, odd dk
     (1032, 1048, 2049, 1, 8),
