@@ -782,7 +782,7 @@ def main():
         "bound": "mfma", "achieved": flops_per_launch / launch_s / 1e12, "peak": PEAK_TFLOPS[w.storage],
         "unit": "TFLOP/s", "frac": flops_per_launch / launch_s / 1e12 / PEAK_TFLOPS[w.storage],
         "traffic": HEADLINE_TRAFFIC_BYTES if head["workload"] == HEADLINE else None,
-        "kernel": "gemm_f32_lds_kernel<A_KMAJOR,B_KMAJOR,false> (fw, ga, gb)" if head["workload"] == HEADLINE
+        "kernel": "gemm_f32_lds_kernel<A_KMAJOR,B_KMAJOR,0> (fw, ga, gb)" if head["workload"] == HEADLINE
                   else "+".join(head["gemm_kernels_first_timestep"]),
         "flops_per_launch": flops_per_launch, "avg_launch_ms": launch_s * 1e3,
     }
