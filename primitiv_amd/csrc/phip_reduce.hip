@@ -202,11 +202,11 @@ __device__ inline typename OP::State walk_packs(const T *p, uint32_t first, uint
 // A long reduction may be cut into `splits` ranges of `chunk` positions, each
 // reduced by its own workgroup into partial[(o*splits + sp)*base + i]. The
 // workgroup that finishes last of a group's ranges (a counter per group tells)
-// merges them in order and writes the results; without counters a second
-// launch (reduce_finish_kernel) does.  splits == 1 writes the result directly.
+// merges them in order and writes the results.  splits == 1 writes the result
+// directly.
 struct Split {
   uint32_t splits, chunk;
-  uint32_t *tickets;   // splits > 1: one zeroed counter per group of outputs, left zeroed; or null
+  uint32_t *tickets;   // splits > 1: one zeroed counter per group of outputs, left zeroed
 };
 
 // Partial states travel between workgroups, which may sit on different L2s:
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(kBlock) void reduce_block_kernel(const T *x, T *y, 
       __syncthreads();
     }
     if (threadIdx.x == 0) finish<T, OP, EMIT>(part[0], partial, sp, r, y, index_out, gy, gx, o, i, base, n);
-    if (sp.splits > 1 && sp.tickets != nullptr) {
+    if (sp.splits > 1) {
       if (last_of_group(sp.tickets + q, sp.splits, &last) && threadIdx.x == 0)
         merge_ranges<T, OP, EMIT>(partial, sp.splits, y, index_out, gy, gx, o, i, base, n);
     }
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, 
         finish<T, OP, EMIT>(st[k], partial, sp, r, y, index_out, gy, gx, o, i + k, base, n);
       }
     }
-    if (sp.splits > 1 && sp.tickets != nullptr) {
+    if (sp.splits > 1) {
       if (last_of_group(sp.tickets + t, sp.splits, &last)) {
         const uint32_t i0 = (uint32_t)(t - o * per_o) * TX * V;
         for (uint32_t e = threadIdx.x; e < TX * V && i0 + e < base; e += kBlock)
@@ -425,20 +425,6 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(const T *x, T *y, 
       }
     }
     __syncthreads();
-  }
-}
-
-// Merges the ranges of one output in order: thread per output.
-template <typename T, typename OP, Emit EMIT>
-__global__ __launch_bounds__(kBlock) void reduce_finish_kernel(const typename OP::State *partial, uint32_t splits,
-                                                                T *y, uint32_t *index_out, const T *gy, T *gx,
-                                                                uint32_t base, uint32_t n, size_t outputs) {
-  for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < outputs; q += (size_t)gridDim.x * kBlock) {
-    const size_t o = q / base;
-    const uint32_t i = (uint32_t)(q - o * base);
-    typename OP::State st = partial[(o * splits) * base + i];
-    for (uint32_t r = 1; r < splits; ++r) OP::merge(st, partial[(o * splits + r) * base + i]);
-    emit<T, OP, EMIT>(st, y, index_out, gy, gx, q, o * n * base + i, base, n);
   }
 }
 
@@ -495,12 +481,12 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
   const int cols = wide ? kCols : wide2 ? kHalf : 1;
   const size_t groups = by_block ? outputs : (size_t)((base + tx * cols - 1) / (tx * cols)) * outer;
   Split sp = choose_split(groups, n, by_block ? 1024 : 256, cus);
+  if (groups > (size_t)kTicketSlots) sp = Split{1, n, nullptr};  // a counter per group, or no ranges
   void *block = nullptr;
   if (sp.splits > 1) {
-    const int rc = phip_pool_alloc(ctx, sizeof(State) * outputs * sp.splits, &block, nullptr);
+    const int rc = scratch_alloc(ctx, sizeof(State) * outputs * sp.splits, &block);  // the context's private scratch pool
     if (rc != PHIP_OK) return rc;
-    // the last workgroup of a group merges its ranges when there is a counter per group; else a second launch does
-    if (groups <= (size_t)kTicketSlots) sp.tickets = ctx->tile_tickets;
+    sp.tickets = ctx->tile_tickets;
   }
   State *partial = static_cast<State *>(block);
   const size_t blocks = groups * sp.splits;
@@ -522,11 +508,7 @@ int launch_reduce(phip_ctx *ctx, const T *x, T *y, uint32_t *index_out, const T 
                        gy, gx, partial, sp, base, n, outer);
   }
   if (sp.splits > 1) {
-    if (sp.tickets == nullptr) {
-      hipLaunchKernelGGL((reduce_finish_kernel<T, OP, EMIT>), dim3(blocks_for(outputs, ctx)), dim3(kBlock), 0,
-                         ctx->stream, partial, sp.splits, y, index_out, gy, gx, base, n, outputs);
-    }
-    phip_pool_free(ctx, block);  // the stream is in order: the block may be handed out again behind these launches
+    scratch_free(ctx, block);  // the stream is in order: the block may be handed out again behind this launch
   }
   PHIP_LAUNCH_CHECK();
   return PHIP_OK;
