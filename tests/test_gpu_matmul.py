@@ -559,6 +559,9 @@ BIG_H16 = [  # di, dj, dk, ba, bb
     (1024, 264, 1024, 1, 1),
     (1032, 192, 776, 1, 1),
     (776, 3080, 760, 1, 1),
+    # 48 K tiles; 3 samples of 16 tiles summed into a shared operand's gradient
+    (776, 3072, 760, 1, 1),
+    (1024, 512, 1024, 1, 3),
     # one large shared a against at least 16 Ki columns: the forward product runs on a transposed copy of a
     # (both operands then contiguous along k); ragged in every dimension, K tail, odd dk
     (1032, 1048, 2049, 1, 8),
