@@ -389,6 +389,33 @@ def test_half_storage_aligned_copies_match_oracle(dev16):
     _aligned_copies(dev16, False)
 
 
+@pytest.mark.parametrize("dims,batch,dim", [([256, 4096], 1, 1), ([20000], 3, 0), ([130, 3000], 2, 1), ([16, 70000], 1, 1)])
+def test_long_reductions_cut_into_ranges_are_reproducible(dev, dims, batch, dim):
+    # few outputs over a long dimension: the dimension is cut into ranges reduced by different workgroups, and the
+    # one that finishes last merges them in order - the same bits whichever that is
+    rng = np.random.default_rng(dims[0] + batch)
+    n = int(np.prod(dims)) * batch
+    x = rng.standard_normal(n).astype(np.float32)
+    tx = dev.new_tensor_by_vector(S(dims, batch), x)
+    for op in ("sum", "logsumexp", "max"):
+        first = dev.reduce_fw(op, tx, dim).to_vector()
+        want = oracle.reduce_fw(op, x, dims, batch, dim)
+        if op == "max":
+            assert np.array_equal(first, want)
+        elif op == "logsumexp":
+            assert np.allclose(first, want, rtol=1e-5, atol=1e-4)
+        else:
+            # against the sum in float64; an fp32 sum of n values of unit variance, in whatever order, is good to
+            # a few times 1e-7 n at the very worst
+            exact = np.moveaxis(x.astype(np.float64).reshape([batch] + dims[::-1]), len(dims) - dim, -1).sum(-1).reshape(-1)
+            assert np.max(np.abs(first - exact)) <= 3e-7 * dims[dim]
+        for _ in range(10):
+            assert np.array_equal(dev.reduce_fw(op, tx, dim).to_vector(), first)
+    idx = oracle.arg_extremum("max", x, dims, batch, dim)
+    for _ in range(5):
+        assert np.array_equal(dev.arg_extremum("max", tx, dim), idx)
+
+
 @pytest.mark.parametrize("dims,batch,dim", [([130, 517], 2, 1), ([256, 40, 3], 1, 1), ([129, 300], 1, 1), ([64, 1031], 3, 0),
                                             ([260, 300], 2, 1), ([516, 70, 2], 1, 1), ([512, 520], 1, 0), ([520, 300], 2, 0),
                                             ([1032, 515], 1, 0)])
