@@ -599,6 +599,20 @@ def test_large_tile_h16(dev16, devbf16, which, di, dj, dk, ba, bb):
         assert norm_rel_err(got, ref) <= ulp
 
 
+def test_mid_tiles_take_four_stages_h16(dev16):
+    # at most one 128 x 128 tile per CU: the launch with four LDS stages; more tiles than CUs: two stages
+    rng = np.random.default_rng(3)
+    for (di, dj, dk), want in (((1536, 1536, 1536), "h16_lds128_deep"), ((1024, 192, 1024), "h16_lds128"),
+                               ((2304, 1024, 2048), "h16_lds128")):
+        a = dev16.new_tensor_by_vector(pa.Shape([di, dj]), rng.standard_normal(di * dj).astype(np.float32))
+        b = dev16.new_tensor_by_vector(pa.Shape([dj, dk]), rng.standard_normal(dj * dk).astype(np.float32))
+        dev16.gemm_trace(True)
+        y = dev16.matmul_fw(a, b)
+        assert dev16.gemm_trace(False) == [want], (di, dj, dk)
+        ref = a.to_vector().astype(np.float64).reshape(dj, di).T @ b.to_vector().astype(np.float64).reshape(dk, dj).T
+        assert norm_rel_err(y.to_vector(), ref.T.reshape(-1)) <= H16_TOL
+
+
 # few output tiles over a long K on the 16-bit devices: the K range is cut between
 # workgroups that leave fp32 partial tiles, summed in order by a second launch
 # (gb of the first two shapes, the forward product of the third)
