@@ -236,6 +236,54 @@ def test_drawn_dimensions_all_devices(dev, dev16, devbf16, seed):
             assert norm_rel_err(gb, stored[4] + dgb) <= tol, "gb " + tag
 
 
+def _drawn_shape(rng, kind):
+    if kind == 0:   # small, any alignment
+        return [int(rng.integers(1, 300)) for _ in range(3)]
+    if kind == 1:   # few columns against a long or tall operand: the per-timestep shapes
+        return [int(rng.integers(1, 4000)), int(rng.integers(1, 3000)), int(rng.integers(1, 130))]
+    if kind == 2:   # short K: rank-K updates
+        return [int(rng.integers(64, 3000)), int(rng.integers(1, 100)), int(rng.integers(64, 2000))]
+    if kind == 3:   # mid-size, multiples of 4: the tile kernels and their split / mixed launches
+        return [int(rng.integers(16, 500)) * 4 for _ in range(3)]
+    if kind == 4:   # few outputs over a very long K
+        return [int(rng.integers(1, 200)), int(rng.integers(2000, 40000)), int(rng.integers(1, 200))]
+    return [int(rng.integers(100, 1800)) for _ in range(3)]   # mid-size, any alignment
+
+
+@pytest.mark.parametrize("seed", range(2))
+def test_drawn_shape_classes_all_devices(dev, dev16, devbf16, seed):
+    # Whole shapes drawn class by class (where the draw above draws each axis on its own), each in a drawn
+    # batch case, on the fp32 device in both accumulation modes and on both 16-bit devices, against
+    # float64 numpy on the values each device stores.
+    rng = np.random.default_rng(7000 + seed)
+    det = pa.HIP(0)
+    det.set_deterministic(True)
+    for it in range(30):
+        di, dj, dk = _drawn_shape(rng, it % 6)
+        ba, bb = [(1, 1), (1, int(rng.integers(2, 6))), (int(rng.integers(2, 6)), 1), (3, 3)][int(rng.integers(0, 4))]
+        bs = max(ba, bb)
+        while di * dj * dk * bs > 2e9:
+            di, dk = max(1, di // 2), max(1, dk // 2)
+        a = rng.standard_normal(di * dj * ba).astype(np.float32)
+        b = rng.standard_normal(dj * dk * bb).astype(np.float32)
+        gy = rng.standard_normal(di * dk * bs).astype(np.float32)
+        ga0 = rng.standard_normal(a.size).astype(np.float32)
+        gb0 = rng.standard_normal(b.size).astype(np.float32)
+        for d, tol in ((dev, F32_TOL), (det, F32_TOL), (dev16, H16_TOL), (devbf16, H16_TOL)):
+            stored = [d.new_tensor_by_vector(pa.Shape(dims, n), v).to_vector().astype(np.float64)
+                      for dims, n, v in (([di, dj], ba, a), ([dj, dk], bb, b), ([di, dk], bs, gy),
+                                         ([di, dj], ba, ga0), ([dj, dk], bb, gb0))]
+            y, ga, gb = _fw_bw(d, a, b, gy, ga0, gb0, di, dj, dk, ba, bb)
+            ry = np_matmul_fw(stored[0], stored[1], di, dj, dk, ba, bb)
+            dga, dgb = np_matmul_bw(stored[0], stored[1], stored[2], di, dj, dk, ba, bb)
+            tag = "%s%s draw %d shape (%d,%d,%d) batch (%d,%d)" % (type(d).__name__, " deterministic" if d is det else "",
+                                                                   it, di, dj, dk, ba, bb)
+            assert norm_rel_err(y, ry) <= tol, "y " + tag
+            assert norm_rel_err(ga, stored[3] + dga) <= tol, "ga " + tag
+            assert norm_rel_err(gb, stored[4] + dgb) <= tol, "gb " + tag
+    det.close()
+
+
 # shapes that reach the fp32 128x128x32 global-to-LDS kernel (>= one tile per CU)
 # with ragged edges in every dimension (multiples of 4, not of 128 / 32)
 BIG_F32 = [  # di, dj, dk, ba, bb
